@@ -1,0 +1,290 @@
+#!/usr/bin/env python3
+"""Throughput of the fusion-buffer hot path on one MI355X.
+
+One "step" is one pass of the hot path over one batch of synthetic gradients.
+The headline workload is the fusion stress configuration: 1,024 fp32 tensors
+with element counts log-uniform in [256, 65536] (seed 3), values U(-1,1)
+(seed 4), packed into a 64 MiB fusion buffer with prescale 0.125 and unpacked
+again.  Inputs are resident in HBM before the timed region starts.
+
+Prints ONE JSON line.  `value` is algorithmic GB/s of the whole step
+(pack = P_in + P_buf, unpack = P_buf + P_out); `roofline` prices the dominant
+kernel (the scaled pack) against the 8 TB/s HBM peak from its average launch
+duration measured with HIP events on the stream it runs on; `cpu_baseline` is
+the CPU oracle (a restatement of the reference's CPU path) timed on one host
+core over the same workload; `extra` carries the other pipelines (ResNet-50
+cycle with a peer reduce, BERT-large fp16-compressed with 7 peers, Adasum,
+GPT-2 XL streamed on two streams).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--kernel-only", action="store_true",
+                    help="only launch the dominant kernel (for rocprofv3 runs)")
+    return ap.parse_args()
+
+
+def timed(fn, sync, steps, warmup):
+    """Wall time of `steps` calls of fn bracketed by synchronisation on both sides."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    sync()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def event_timed(fn, stream, steps, warmup):
+    """Average stream time per call of fn, from HIP events recorded on `stream`."""
+    from horovod_amd import Timer
+    for _ in range(warmup):
+        fn()
+    stream.synchronize()
+    t = Timer()
+    t.start(stream)
+    for _ in range(steps):
+        fn()
+    t.stop(stream)
+    ms = t.elapsed_ms()
+    t.destroy()
+    return ms / steps * 1e-3
+
+
+class DeviceSet:
+    """Gradient tensors carved out of one device allocation at 256-byte aligned offsets."""
+
+    def __init__(self, counts, elem_size, fill):
+        import torch
+        self.counts = counts
+        self.es = elem_size
+        offs, cur = [], 0
+        for c in counts:
+            offs.append(cur)
+            cur += (c * elem_size + 255) // 256 * 256
+        self.offs = offs
+        self.nbytes = max(cur, 256)
+        self.dev = fill(self.nbytes)
+        torch.cuda.synchronize()
+        self.ptrs = [self.dev.data_ptr() + o for o in offs]
+
+
+def stress_workload():
+    import torch
+    from horovod_amd import workloads as W
+    counts = W.stress_counts(seed=3)
+    rng = np.random.default_rng(4)
+    host = np.zeros(sum((c * 4 + 255) // 256 * 256 for c in counts), np.uint8)
+
+    def fill(nbytes):
+        off = 0
+        for c in counts:
+            host[off:off + 4 * c] = rng.uniform(-1, 1, c).astype(np.float32).view(np.uint8)
+            off += (c * 4 + 255) // 256 * 256
+        return torch.from_numpy(host).cuda()
+
+    src = DeviceSet(counts, 4, fill)
+    dst = DeviceSet(counts, 4, lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
+    return counts, host, src, dst
+
+
+def cpu_baseline_stress(counts, host, budget_s=12.0):
+    """The reference CPU sequence (ops/gloo_operations.cc:118-170) on one core:
+    memcpy pack, in-place ScaleBuffer(0.125), memcpy unpack."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_util
+    from ctypes import c_double, c_int, c_int64, c_void_p
+    orc = oracle_util.Oracle()
+    L = orc.lib
+    offs, cur = [], 0
+    for c in counts:
+        offs.append(cur)
+        cur += (c * 4 + 255) // 256 * 256
+    out = np.zeros_like(host)
+    n = len(counts)
+    tptr = (c_void_p * n)(*[host.ctypes.data + o for o in offs])
+    optr = (c_void_p * n)(*[out.ctypes.data + o for o in offs])
+    nb = np.array([4 * c for c in counts], np.int64)
+    payload = int(nb.sum())
+    buf = np.zeros(payload + 64, np.uint8)
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        L.orc_pack(tptr, c_void_p(nb.ctypes.data), c_int(n), c_void_p(buf.ctypes.data))
+        L.orc_scale_buffer(c_void_p(buf.ctypes.data), c_void_p(buf.ctypes.data), c_int64(payload // 4),
+                           c_double(0.125), c_int(oracle_util.F32))
+        L.orc_unpack(c_void_p(buf.ctypes.data), optr, c_void_p(nb.ctypes.data), c_int(n))
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt > budget_s or reps >= 200:
+            break
+    gbs = 4 * payload * reps / dt / 1e9
+    return {"value": round(gbs, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "%d repetitions of the same 1,024-tensor workload (memcpy pack, in-place ScaleBuffer 0.125, "
+                      "memcpy unpack; 4P algorithmic bytes each) in %.1f s; host has %d cores"
+                      % (reps, dt, os.cpu_count())}
+
+
+def extras(steps, warmup):
+    """The other pipelines, each as algorithmic GB/s and fraction of the HBM peak."""
+    import torch
+    from horovod_amd import AdasumPlan, DTYPE, Stream, workloads as W
+    from horovod_amd.pipeline import AllreducePipeline
+    out = {}
+    g = torch.Generator(device="cuda")
+
+    def randn(nbytes, dtype, std, seed):
+        g.manual_seed(seed)
+        n = nbytes // torch.empty(0, dtype=dtype).element_size()
+        return (torch.randn(n, generator=g, device="cuda", dtype=torch.float32) * std).to(dtype).view(torch.uint8)
+
+    def run_pipeline(name, shapes, tdtype, bdtype, std, peers, fraction, streams, kway=True, steps_=steps):
+        tt = {DTYPE["float32"]: torch.float32, DTYPE["float16"]: torch.float16}
+        es = 4 if tdtype == DTYPE["float32"] else 2
+        counts = [W.numel(s) for s in shapes]
+        src = DeviceSet(counts, es, lambda n: randn(n, tt[tdtype], std, 1))
+        dst = DeviceSet(counts, es, lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
+        pipe = AllreducePipeline(src.ptrs, dst.ptrs, counts, tdtype, bdtype, num_streams=streams)
+        bs = 4 if pipe.buffer_dtype == DTYPE["float32"] else 2
+        max_elems = max(c.buffer_elems for c in pipe.cycles)
+        peer_bufs = []
+        for p in range(peers):
+            nb = int(max_elems * fraction) * bs + 256
+            peer_bufs.append(randn((nb + 255) // 256 * 256, tt[pipe.buffer_dtype], std, 100 + p))
+        torch.cuda.synchronize()
+        fn = lambda: pipe.run(0.125, 1.0, (lambda ci, p: peer_bufs[p].data_ptr()) if peers else None,
+                              peers, fraction, kway)
+        sec = timed(fn, pipe.synchronize, steps_, max(2, warmup // 4))
+        ab = pipe.algorithmic_bytes(peers, fraction, kway)
+        out[name] = {"GB/s": round(ab / sec / 1e9, 1), "frac_of_hbm_peak": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4),
+                     "ms": round(sec * 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1), "cycles": len(pipe.cycles),
+                     "streams": streams, "peers": peers, "reduce": "k-way" if kway else "per-peer"}
+        pipe.destroy()
+        del src, dst, peer_bufs
+        torch.cuda.empty_cache()
+
+    F32, F16 = DTYPE["float32"], DTYPE["float16"]
+    run_pipeline("resnet50_fp32_pack_scale_reduce_unpack", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0, 1)
+    run_pipeline("bert_large_fp32_to_fp16_7peers_eighth_chunk", W.bert_large_shapes(), F32, F16, 1e-4, 7, 0.125, 1,
+                 steps_=max(5, steps // 10))
+    run_pipeline("gpt2_xl_fp16_two_streams", W.gpt2_xl_shapes(), F16, F16, 1e-3, 1, 1.0, 2,
+                 steps_=max(3, steps // 40))
+
+    # Adasum combine: two fp32 vectors of 2^25 elements, 64 layers, per-layer correlation 0.3
+    n = 1 << 25
+    counts = W.adasum_layer_counts(n, 64, seed=13)
+    g.manual_seed(14)
+    a = torch.randn(n, generator=g, device="cuda", dtype=torch.float32)
+    g.manual_seed(15)
+    b = 0.3 * a + (1 - 0.09) ** 0.5 * torch.randn(n, generator=g, device="cuda", dtype=torch.float32)
+    a0 = a.clone()
+    plan = AdasumPlan(counts, F32)
+    s = Stream()
+    torch.cuda.synchronize()
+
+    def combine():
+        plan.combine(a.data_ptr(), b.data_ptr(), s)
+
+    # the combine rewrites a; its cost does not depend on the values, which stay finite:
+    # coefficients are <= 1 in magnitude for positively correlated pairs
+    sec = event_timed(combine, s, max(5, steps // 4), 3)
+    ab = 5 * n * 4
+    out["adasum_fp32_2x32M_64layers"] = {"GB/s": round(ab / sec / 1e9, 1),
+                                         "frac_of_hbm_peak": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4),
+                                         "ms": round(sec * 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1)}
+    plan.destroy()
+    s.destroy()
+    del a, b, a0
+    return out
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU's share of the hot path: this build has no inter-GPU collectives, "
+              "run it with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    import horovod_amd
+    from horovod_amd import DTYPE, FusionPlan, Stream
+    horovod_amd.lib()  # fails loudly if the HIP library is not built
+
+    counts, host, src, dst = stress_workload()
+    F32 = DTYPE["float32"]
+    plan = FusionPlan(src.ptrs, dst.ptrs, counts, F32)
+    fb = torch.empty(plan.buffer_len, dtype=torch.uint8, device="cuda")
+    stream = Stream()
+    payload = 4 * sum(counts)
+    torch.cuda.synchronize()
+
+    def pack():
+        plan.pack(fb.data_ptr(), 0.125, stream)
+
+    def step():
+        plan.pack(fb.data_ptr(), 0.125, stream)
+        plan.unpack(fb.data_ptr(), 1.0, stream)
+
+    if args.kernel_only:
+        for _ in range(args.warmup + args.steps):
+            pack()
+        stream.synchronize()
+        return
+
+    sec = timed(step, stream.synchronize, args.steps, args.warmup)
+    value = 4 * payload / sec / 1e9
+
+    ksec = event_timed(pack, stream, args.steps, args.warmup)
+    achieved = 2 * payload / ksec / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "kernel": "xfer_k<Scale<float,float>, pack>", "launch_us": round(ksec * 1e6, 2),
+                "algorithmic_bytes_per_launch": 2 * payload, "workgroups": plan.num_chunks}
+
+    result = {
+        "metric": "achieved HBM GB/s (% of 8 TB/s) for fused pack+scale+reduce+unpack; Adasum GB/s",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "fusion stress: 1,024 fp32 tensors, log-uniform 256..65,536 elements (seed 3), "
+                               "U(-1,1) (seed 4); pack with prescale 0.125 into a 64 MiB fusion buffer, unpack",
+                   "tensors": len(counts), "payload_bytes": payload, "buffer_len": plan.buffer_len,
+                   "algorithmic_bytes_per_step": 4 * payload},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "roofline": roofline,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline_stress(counts, host)
+    plan.destroy()
+    del fb, src, dst
+    torch.cuda.empty_cache()
+    if not args.no_extra:
+        result["extra"] = extras(args.steps, args.warmup)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,483 @@
+// adasum.hip -- Adasum's pairwise combine on one device: per-layer dot
+// product and squared norms accumulated in double, the coefficient formula,
+// and the fused scaled add.  gfx950 only.
+//
+// Follows Adasum<Comm>::FusedPairwiseReduceWithComm, ops/adasum/adasum.h:344-410,
+// with ComputeDotAndNormSqrds (:413-426) and ScaledAdd (:429-435); in the
+// reference all of it runs on the host.
+//
+// Pass 1 (dot_partials_k): one workgroup per chunk of a layer.  Each lane
+// streams 16-byte pieces of a and b, widens to double and keeps two
+// independent fma chains per sum; lanes combine with wave64 shuffles, the four
+// wavefronts through LDS, and the workgroup writes one {dot, |a|^2, |b|^2}
+// triple.  Pass 1b (finalize_k): one workgroup per layer adds that layer's
+// triples in a fixed order and evaluates the coefficients.  No floating-point
+// atomics anywhere, so results are identical from run to run.
+// Pass 2 (scaled_add_k): one workgroup per chunk, a = ca*a + cb*b in double,
+// rounded once.
+//
+// Products of two fp32 (or fp16) values are exact in double, so only the
+// order of the double additions differs from the reference's sequential
+// loop.  Bandwidth-bound: 3 double fmas per 8 bytes read in pass 1.
+#include <cfloat>
+#include <cmath>
+#include <list>
+#include <mutex>
+
+#include "internal.h"
+#include "vecmem.h"
+
+namespace hvdhip {
+namespace {
+
+// Layer table entry, stored in a Seg: off = first element of the layer,
+// n = its element count, output = index of its first chunk (= first partial
+// triple), tensor = number of chunks.
+
+struct Triple {
+  double d, a, b;
+};
+
+__device__ __forceinline__ Triple wg_reduce(Triple t) {
+  // wave64 tree, then the four wavefronts in order through LDS
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    t.d += __shfl_down(t.d, o, 64);
+    t.a += __shfl_down(t.a, o, 64);
+    t.b += __shfl_down(t.b, o, 64);
+  }
+  __shared__ double red[3][kWG / 64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    red[0][wave] = t.d;
+    red[1][wave] = t.a;
+    red[2][wave] = t.b;
+  }
+  __syncthreads();
+  Triple r = {0., 0., 0.};
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int w = 0; w < kWG / 64; ++w) {
+      r.d += red[0][w];
+      r.a += red[1][w];
+      r.b += red[2][w];
+    }
+  }
+  return r;  // valid in thread 0
+}
+
+constexpr int kUnroll = 4;
+
+template <typename T>
+__global__ __launch_bounds__(kWG) void dot_partials_k(const Seg* __restrict__ layers,
+                                                      const Chunk* __restrict__ chunks,
+                                                      const T* __restrict__ a,
+                                                      const T* __restrict__ b,
+                                                      uint32_t chunk_units,
+                                                      double* __restrict__ partials) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  typedef Arr<T, VEC> V;
+  const Chunk c = chunks[blockIdx.x];
+  const Seg L = layers[c.seg];
+  const uint64_t start = (uint64_t)c.idx * chunk_units;
+  const uint64_t left = L.n - start;
+  const uint32_t n = left < chunk_units ? (uint32_t)left : chunk_units;
+  gptr<const T> pa = as_global(a + L.off + start);
+  gptr<const T> pb = as_global(b + L.off + start);
+  const uint32_t nv = n / VEC;
+  double d0 = 0., d1 = 0., a0 = 0., a1 = 0., b0 = 0., b1 = 0.;
+  uint32_t v = threadIdx.x;
+  for (; v + (kUnroll - 1) * kWG < nv; v += kUnroll * kWG) {
+    V x[kUnroll], y[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      x[u] = ldv<T, VEC>(pa + (size_t)(v + u * kWG) * VEC);
+      y[u] = ldv<T, VEC>(pb + (size_t)(v + u * kWG) * VEC);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+      for (int j = 0; j < VEC; j += 2) {
+        const double p = (double)x[u].v[j], q = (double)y[u].v[j];
+        d0 = fma(p, q, d0);
+        a0 = fma(p, p, a0);
+        b0 = fma(q, q, b0);
+        if (j + 1 < VEC) {
+          const double r = (double)x[u].v[j + 1], s = (double)y[u].v[j + 1];
+          d1 = fma(r, s, d1);
+          a1 = fma(r, r, a1);
+          b1 = fma(s, s, b1);
+        }
+      }
+    }
+  }
+  for (; v < nv; v += kWG) {
+    const V x = ldv<T, VEC>(pa + (size_t)v * VEC), y = ldv<T, VEC>(pb + (size_t)v * VEC);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const double p = (double)x.v[j], q = (double)y.v[j];
+      d0 = fma(p, q, d0);
+      a0 = fma(p, p, a0);
+      b0 = fma(q, q, b0);
+    }
+  }
+  const uint32_t t = nv * VEC + threadIdx.x;
+  if (t < n) {
+    const double p = (double)pa[t], q = (double)pb[t];
+    d1 = fma(p, q, d1);
+    a1 = fma(p, p, a1);
+    b1 = fma(q, q, b1);
+  }
+  Triple r = wg_reduce(Triple{d0 + d1, a0 + a1, b0 + b1});
+  if (threadIdx.x == 0) {
+    partials[3 * (uint64_t)blockIdx.x + 0] = r.d;
+    partials[3 * (uint64_t)blockIdx.x + 1] = r.a;
+    partials[3 * (uint64_t)blockIdx.x + 2] = r.b;
+  }
+}
+
+// One workgroup per layer: sums the layer's partial triples in a fixed order,
+// stores {dot, |a|^2, |b|^2} and the coefficients of adasum.h:397-404.
+__global__ __launch_bounds__(kWG) void finalize_k(const Seg* __restrict__ layers,
+                                                  const double* __restrict__ partials,
+                                                  double* __restrict__ normdots,
+                                                  double* __restrict__ coeffs, double guard) {
+  const Seg L = layers[blockIdx.x];
+  const uint64_t first = L.output, count = L.tensor;
+  Triple t = {0., 0., 0.};
+  for (uint64_t i = threadIdx.x; i < count; i += kWG) {
+    t.d += partials[3 * (first + i) + 0];
+    t.a += partials[3 * (first + i) + 1];
+    t.b += partials[3 * (first + i) + 2];
+  }
+  Triple r = wg_reduce(t);
+  if (threadIdx.x == 0) {
+    normdots[3 * (uint64_t)blockIdx.x + 0] = r.d;
+    normdots[3 * (uint64_t)blockIdx.x + 1] = r.a;
+    normdots[3 * (uint64_t)blockIdx.x + 2] = r.b;
+    double ca = 1., cb = 1.;
+    if (r.a >= guard) ca = 1.0 - r.d / r.a * 0.5;
+    if (r.b >= guard) cb = 1.0 - r.d / r.b * 0.5;
+    coeffs[2 * (uint64_t)blockIdx.x + 0] = ca;
+    coeffs[2 * (uint64_t)blockIdx.x + 1] = cb;
+  }
+}
+
+// ScaledAdd<T>, adasum.h:429-435: operands widened to double, one rounding.
+template <typename T>
+struct Axpby {
+  static __device__ __forceinline__ T f(double ca, T a, double cb, T b) {
+    return (T)fma(ca, (double)a, cb * (double)b);
+  }
+};
+// ScaledAddfp16, adasum.h:482-500: float coefficients, t = ca*a rounded to
+// fp32, r = fma(cb, b, t), rounded to half.
+template <>
+struct Axpby<half_t> {
+  static __device__ __forceinline__ half_t f(double ca, half_t a, double cb, half_t b) {
+    const float t = __fmul_rn((float)ca, (float)a);
+    return (half_t)__fmaf_rn((float)cb, (float)b, t);
+  }
+};
+
+template <typename T>
+__global__ __launch_bounds__(kWG) void scaled_add_k(const Seg* __restrict__ layers,
+                                                    const Chunk* __restrict__ chunks, T* a,
+                                                    const T* __restrict__ b,
+                                                    uint32_t chunk_units,
+                                                    const double* __restrict__ coeffs,
+                                                    double ca_arg, double cb_arg) {
+  // coeffs == nullptr: every layer uses the by-value pair (ca_arg, cb_arg).
+  constexpr int VEC = 16 / (int)sizeof(T);
+  typedef Arr<T, VEC> V;
+  const Chunk c = chunks[blockIdx.x];
+  const Seg L = layers[c.seg];
+  const double ca = coeffs ? coeffs[2 * (uint64_t)c.seg] : ca_arg;
+  const double cb = coeffs ? coeffs[2 * (uint64_t)c.seg + 1] : cb_arg;
+  const uint64_t start = (uint64_t)c.idx * chunk_units;
+  const uint64_t left = L.n - start;
+  const uint32_t n = left < chunk_units ? (uint32_t)left : chunk_units;
+  gptr<T> pa = as_global(a + L.off + start);
+  gptr<const T> pb = as_global(b + L.off + start);
+  const uint32_t nv = n / VEC;
+  uint32_t v = threadIdx.x;
+  for (; v + (kUnroll - 1) * kWG < nv; v += kUnroll * kWG) {
+    V x[kUnroll], y[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      x[u] = ldv<T, VEC>(pa + (size_t)(v + u * kWG) * VEC);
+      y[u] = ldv<T, VEC>(pb + (size_t)(v + u * kWG) * VEC);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) x[u].v[j] = Axpby<T>::f(ca, x[u].v[j], cb, y[u].v[j]);
+      stv<T, VEC>(pa + (size_t)(v + u * kWG) * VEC, x[u]);
+    }
+  }
+  for (; v < nv; v += kWG) {
+    V x = ldv<T, VEC>(pa + (size_t)v * VEC);
+    const V y = ldv<T, VEC>(pb + (size_t)v * VEC);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) x.v[j] = Axpby<T>::f(ca, x.v[j], cb, y.v[j]);
+    stv<T, VEC>(pa + (size_t)v * VEC, x);
+  }
+  const uint32_t t = nv * VEC + threadIdx.x;
+  if (t < n) pa[t] = Axpby<T>::f(ca, pa[t], cb, pb[t]);
+}
+
+}  // namespace
+}  // namespace hvdhip
+
+using namespace hvdhip;
+
+struct hvdhip_adasum_plan {
+  int nlayers = 0;
+  int dtype = 0;
+  int64_t total = 0;
+  DevTables tables;
+  double* results = nullptr;  // one allocation: partials | normdots | coeffs
+  double* partials = nullptr;
+  double* normdots = nullptr;
+  double* coeffs = nullptr;
+};
+
+namespace {
+
+int plan_dot_norms(hvdhip_adasum_plan* p, const void* a, const void* b, hipStream_t s) {
+  if (p->nlayers == 0) return 0;
+  const DevTables& t = p->tables;
+  if (t.nchunks > 0) {
+    switch (p->dtype) {
+    case HVDHIP_FLOAT16:
+      hipLaunchKernelGGL((dot_partials_k<half_t>), dim3(t.nchunks), dim3(kWG), 0, s, t.segs, t.chunks,
+                         static_cast<const half_t*>(a), static_cast<const half_t*>(b), t.chunk_units,
+                         p->partials);
+      break;
+    case HVDHIP_FLOAT32:
+      hipLaunchKernelGGL((dot_partials_k<float>), dim3(t.nchunks), dim3(kWG), 0, s, t.segs, t.chunks,
+                         static_cast<const float*>(a), static_cast<const float*>(b), t.chunk_units,
+                         p->partials);
+      break;
+    default:
+      hipLaunchKernelGGL((dot_partials_k<double>), dim3(t.nchunks), dim3(kWG), 0, s, t.segs, t.chunks,
+                         static_cast<const double*>(a), static_cast<const double*>(b), t.chunk_units,
+                         p->partials);
+      break;
+    }
+    HVDHIP_CHECK_LAUNCH("dot_partials_k");
+  }
+  hipLaunchKernelGGL(finalize_k, dim3((uint32_t)p->nlayers), dim3(kWG), 0, s, t.segs, p->partials,
+                     p->normdots, p->coeffs, std::sqrt(DBL_MIN));
+  HVDHIP_CHECK_LAUNCH("finalize_k");
+  return 0;
+}
+
+// coeffs == nullptr selects the by-value pair (ca, cb) for every layer.
+int plan_scaled_add(hvdhip_adasum_plan* p, void* a, const void* b, const double* coeffs,
+                    double ca, double cb, hipStream_t s) {
+  const DevTables& t = p->tables;
+  if (t.nchunks == 0) return 0;
+  switch (p->dtype) {
+  case HVDHIP_FLOAT16:
+    hipLaunchKernelGGL((scaled_add_k<half_t>), dim3(t.nchunks), dim3(kWG), 0, s, t.segs, t.chunks,
+                       static_cast<half_t*>(a), static_cast<const half_t*>(b), t.chunk_units, coeffs, ca, cb);
+    break;
+  case HVDHIP_FLOAT32:
+    hipLaunchKernelGGL((scaled_add_k<float>), dim3(t.nchunks), dim3(kWG), 0, s, t.segs, t.chunks,
+                       static_cast<float*>(a), static_cast<const float*>(b), t.chunk_units, coeffs, ca, cb);
+    break;
+  default:
+    hipLaunchKernelGGL((scaled_add_k<double>), dim3(t.nchunks), dim3(kWG), 0, s, t.segs, t.chunks,
+                       static_cast<double*>(a), static_cast<const double*>(b), t.chunk_units, coeffs, ca, cb);
+    break;
+  }
+  HVDHIP_CHECK_LAUNCH("scaled_add_k");
+  return 0;
+}
+
+int check_vectors(const hvdhip_adasum_plan* p, const void* a, const void* b) {
+  if (!p) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "plan is NULL");
+  if (p->total > 0) {
+    if (!a || !b) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "a or b is NULL");
+    if (((uintptr_t)a | (uintptr_t)b) % (uintptr_t)dtype_size(p->dtype))
+      return fail(HVDHIP_ERR_INVALID_ARGUMENT, "a or b is not aligned to its element size");
+  }
+  return 0;
+}
+
+// Single-layer plans for the Dispatch* entry points, keyed by (count, dtype).
+struct OneLayerCache {
+  std::mutex mu;
+  std::list<hvdhip_adasum_plan*> lru;
+};
+OneLayerCache& one_layer_cache() {
+  static OneLayerCache* c = new OneLayerCache();
+  return *c;
+}
+constexpr size_t kOneLayerCapacity = 256;
+
+int one_layer_plan(int count, int dtype, hvdhip_adasum_plan** out) {
+  OneLayerCache& c = one_layer_cache();
+  std::lock_guard<std::mutex> g(c.mu);
+  for (auto it = c.lru.begin(); it != c.lru.end(); ++it) {
+    if ((*it)->total == count && (*it)->dtype == dtype) {
+      c.lru.splice(c.lru.begin(), c.lru, it);
+      *out = c.lru.front();
+      return 0;
+    }
+  }
+  hvdhip_adasum_plan* p = nullptr;
+  int rc = hvdhip_adasum_plan_create(&count, 1, dtype, &p);
+  if (rc) return rc;
+  if (c.lru.size() >= kOneLayerCapacity) {
+    hvdhip_adasum_plan_destroy(c.lru.back());
+    c.lru.pop_back();
+  }
+  c.lru.push_front(p);
+  *out = p;
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int hvdhip_adasum_plan_create(const int* tensor_counts, int nlayers, int dtype,
+                              hvdhip_adasum_plan** plan) {
+  if (!plan) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "plan is NULL");
+  *plan = nullptr;
+  if (nlayers < 0 || (nlayers > 0 && !tensor_counts)) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "bad tensor_counts");
+  if (dtype != HVDHIP_FLOAT16 && dtype != HVDHIP_FLOAT32 && dtype != HVDHIP_FLOAT64)
+    return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE, "Adasum supports FLOAT16, FLOAT32 and FLOAT64, not dtype %d", dtype);
+  const uint32_t chunk_units = chunk_bytes() / (uint32_t)dtype_size(dtype);
+  std::vector<Seg> layers((size_t)nlayers);
+  uint64_t off = 0, first = 0;
+  for (int i = 0; i < nlayers; ++i) {
+    if (tensor_counts[i] < 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "tensor_counts[%d] is negative", i);
+    const uint64_t n = (uint64_t)tensor_counts[i];
+    const uint64_t c = (n + chunk_units - 1) / chunk_units;
+    layers[(size_t)i] = Seg{c, first, off, n};
+    off += n;
+    first += c;
+  }
+  hvdhip_adasum_plan* p = new hvdhip_adasum_plan();
+  p->nlayers = nlayers;
+  p->dtype = dtype;
+  p->total = (int64_t)off;
+  int rc = build_tables(layers, chunk_units, &p->tables);
+  if (rc) {
+    delete p;
+    return rc;
+  }
+  const size_t ndoubles = 3 * (size_t)p->tables.nchunks + 5 * (size_t)nlayers + 8;
+  hipError_t e = hipMalloc(reinterpret_cast<void**>(&p->results), ndoubles * sizeof(double));
+  if (e == hipSuccess) e = hipMemset(p->results, 0, ndoubles * sizeof(double));
+  if (e != hipSuccess) {
+    if (p->results) (void)hipFree(p->results);
+    free_tables(&p->tables);
+    delete p;
+    return fail(e == hipErrorOutOfMemory ? HVDHIP_ERR_OUT_OF_MEMORY : (int)e,
+                "allocating Adasum results failed: %s", hipGetErrorString(e));
+  }
+  p->partials = p->results;
+  p->normdots = p->partials + 3 * (size_t)p->tables.nchunks;
+  p->coeffs = p->normdots + 3 * (size_t)nlayers;
+  *plan = p;
+  return ok();
+}
+
+int hvdhip_adasum_plan_destroy(hvdhip_adasum_plan* plan) {
+  if (!plan) return ok();
+  HVDHIP_CHECK(hipDeviceSynchronize());
+  int rc = free_tables(&plan->tables);
+  if (plan->results) (void)hipFree(plan->results);
+  delete plan;
+  return rc ? rc : ok();
+}
+
+int hvdhip_adasum_dot_norms(hvdhip_adasum_plan* plan, const void* a, const void* b, void* stream) {
+  int rc = check_vectors(plan, a, b);
+  if (rc) return rc;
+  rc = plan_dot_norms(plan, a, b, static_cast<hipStream_t>(stream));
+  return rc ? rc : ok();
+}
+
+int hvdhip_adasum_scaled_add(hvdhip_adasum_plan* plan, void* a, const void* b, void* stream) {
+  int rc = check_vectors(plan, a, b);
+  if (rc) return rc;
+  rc = plan_scaled_add(plan, a, b, plan->coeffs, 0., 0., static_cast<hipStream_t>(stream));
+  return rc ? rc : ok();
+}
+
+int hvdhip_adasum_combine(hvdhip_adasum_plan* plan, void* a, const void* b, void* stream) {
+  int rc = check_vectors(plan, a, b);
+  if (rc) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  rc = plan_dot_norms(plan, a, b, s);
+  if (rc) return rc;
+  rc = plan_scaled_add(plan, a, b, plan->coeffs, 0., 0., s);
+  return rc ? rc : ok();
+}
+
+int hvdhip_adasum_read(hvdhip_adasum_plan* plan, double* normdots, double* coeffs, void* stream) {
+  if (!plan) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "plan is NULL");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (plan->nlayers > 0) {
+    if (normdots)
+      HVDHIP_CHECK(hipMemcpyAsync(normdots, plan->normdots, 3 * (size_t)plan->nlayers * sizeof(double),
+                                  hipMemcpyDeviceToHost, s));
+    if (coeffs)
+      HVDHIP_CHECK(hipMemcpyAsync(coeffs, plan->coeffs, 2 * (size_t)plan->nlayers * sizeof(double),
+                                  hipMemcpyDeviceToHost, s));
+  }
+  HVDHIP_CHECK(hipStreamSynchronize(s));
+  return ok();
+}
+
+int hvdhip_adasum_set_coeffs(hvdhip_adasum_plan* plan, const double* coeffs, void* stream) {
+  if (!plan || (plan->nlayers > 0 && !coeffs)) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "plan or coeffs is NULL");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (plan->nlayers > 0) {
+    HVDHIP_CHECK(hipMemcpyAsync(plan->coeffs, coeffs, 2 * (size_t)plan->nlayers * sizeof(double),
+                                hipMemcpyHostToDevice, s));
+    // The source is caller memory that may change as soon as this returns.
+    HVDHIP_CHECK(hipStreamSynchronize(s));
+  }
+  return ok();
+}
+
+int hvdhip_adasum_dot_and_norm_sqrds(const void* a, const void* b, int dtype, int count,
+                                     double* dot, double* anormsq, double* bnormsq,
+                                     void* stream) {
+  if (!dot || !anormsq || !bnormsq) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "result pointer is NULL");
+  if (count < 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "count is negative");
+  hvdhip_adasum_plan* p = nullptr;
+  int rc = one_layer_plan(count, dtype, &p);
+  if (rc) return rc;
+  rc = check_vectors(p, a, b);
+  if (rc) return rc;
+  rc = plan_dot_norms(p, a, b, static_cast<hipStream_t>(stream));
+  if (rc) return rc;
+  double out[3];
+  rc = hvdhip_adasum_read(p, out, nullptr, stream);
+  if (rc) return rc;
+  *dot = out[0];
+  *anormsq = out[1];
+  *bnormsq = out[2];
+  return ok();
+}
+
+int hvdhip_adasum_dispatch_scaled_add(int dtype, int count, double acoeff, void* a,
+                                      double bcoeff, const void* b, void* stream) {
+  if (count < 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "count is negative");
+  hvdhip_adasum_plan* p = nullptr;
+  int rc = one_layer_plan(count, dtype, &p);
+  if (rc) return rc;
+  rc = check_vectors(p, a, b);
+  if (rc) return rc;
+  rc = plan_scaled_add(p, a, b, nullptr, acoeff, bcoeff, static_cast<hipStream_t>(stream));
+  return rc ? rc : ok();
+}
+
+}  // extern "C"

@@ -1,0 +1,324 @@
+// context.cc -- errors, device, streams, pooled events, timers and the
+// table upload shared by all plans.  Host code only.
+//
+// The stream and event handling follows the member set of the reference's
+// GPUContext::impl (ops/cuda_operations.cc:28-210): one pool of
+// timing-disabled events per (device, stream), filled with 128 events on
+// first use, guarded by a mutex because finalizer threads release events
+// while the background thread acquires them.
+#include <cstdarg>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <utility>
+
+#include "internal.h"
+
+namespace hvdhip {
+
+namespace {
+thread_local std::string g_last_error;
+
+struct EventPools {
+  std::mutex mu;
+  std::map<std::pair<int, hipStream_t>, std::vector<hipEvent_t>> idle;
+  std::map<std::pair<int, hipStream_t>, bool> filled;
+};
+EventPools& pools() {
+  static EventPools* p = new EventPools();  // never destroyed: outlives static teardown
+  return *p;
+}
+constexpr int kPrepopulate = 128;  // N_CUDA_EVENTS_PREPOPULATE, ops/cuda_operations.cc:218
+
+struct Timer {
+  hipEvent_t start;
+  hipEvent_t stop;
+};
+}  // namespace
+
+int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
+
+int ok() {
+  g_last_error.clear();
+  return 0;
+}
+
+uint32_t chunk_bytes() {
+  static uint32_t v = [] {
+    const char* e = getenv("HVDHIP_CHUNK_BYTES");
+    if (e) {
+      long x = strtol(e, nullptr, 10);
+      if (x >= 4096 && x <= (1 << 24) && x % 4096 == 0) return (uint32_t)x;
+    }
+    return kDefaultChunkBytes;
+  }();
+  return v;
+}
+
+int build_tables(const std::vector<Seg>& segs, uint32_t chunk_units, DevTables* out) {
+  if (chunk_units == 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "chunk_units is zero");
+  uint64_t nchunks = 0;
+  for (const Seg& s : segs) {
+    uint64_t c = (s.n + chunk_units - 1) / chunk_units;
+    if (c > 0xffffffffull) return fail(HVDHIP_ERR_TOO_LARGE, "a segment needs more than 2^32 chunks");
+    nchunks += c;
+  }
+  if (nchunks > 0x7fffffffull || segs.size() > 0x7fffffffull)
+    return fail(HVDHIP_ERR_TOO_LARGE, "plan needs %llu workgroups; the limit is 2^31-1",
+                (unsigned long long)nchunks);
+  size_t seg_bytes = (segs.size() * sizeof(Seg) + 255) & ~(size_t)255;
+  size_t chunk_bytes_total = nchunks * sizeof(Chunk);
+  size_t total = seg_bytes + chunk_bytes_total;
+  if (total == 0) total = 256;
+  std::vector<unsigned char> host(total, 0);
+  if (!segs.empty()) memcpy(host.data(), segs.data(), segs.size() * sizeof(Seg));
+  Chunk* hc = reinterpret_cast<Chunk*>(host.data() + seg_bytes);
+  uint64_t k = 0;
+  for (size_t i = 0; i < segs.size(); ++i) {
+    uint64_t c = (segs[i].n + chunk_units - 1) / chunk_units;
+    for (uint64_t j = 0; j < c; ++j) hc[k++] = Chunk{(uint32_t)i, (uint32_t)j};
+  }
+  void* dev = nullptr;
+  hipError_t e = hipMalloc(&dev, total);
+  if (e != hipSuccess)
+    return fail(e == hipErrorOutOfMemory ? HVDHIP_ERR_OUT_OF_MEMORY : (int)e,
+                "hipMalloc of %zu table bytes failed: %s", total, hipGetErrorString(e));
+  e = hipMemcpy(dev, host.data(), total, hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    (void)hipFree(dev);
+    return fail((int)e, "hipMemcpy of plan tables failed: %s", hipGetErrorString(e));
+  }
+  out->alloc = dev;
+  out->segs = reinterpret_cast<Seg*>(dev);
+  out->chunks = reinterpret_cast<Chunk*>(static_cast<unsigned char*>(dev) + seg_bytes);
+  out->nsegs = (uint32_t)segs.size();
+  out->nchunks = (uint32_t)nchunks;
+  out->chunk_units = chunk_units;
+  return 0;
+}
+
+int free_tables(DevTables* t) {
+  if (t->alloc) {
+    HVDHIP_CHECK(hipFree(t->alloc));
+    t->alloc = nullptr;
+  }
+  return 0;
+}
+
+}  // namespace hvdhip
+
+using namespace hvdhip;
+
+extern "C" {
+
+const char* hvdhip_error_string(int code) {
+  if (code == 0) return "success";
+  if (code > 0) return hipGetErrorString((hipError_t)code);
+  switch (code) {
+  case HVDHIP_ERR_INVALID_ARGUMENT: return "invalid argument";
+  case HVDHIP_ERR_UNSUPPORTED_DTYPE: return "data type not supported by this operation";
+  case HVDHIP_ERR_OUT_OF_MEMORY: return "out of device memory";
+  case HVDHIP_ERR_TOO_LARGE: return "size exceeds what one launch can cover";
+  default: return "unknown hvdhip error";
+  }
+}
+
+const char* hvdhip_last_error(void) { return g_last_error.c_str(); }
+
+int64_t hvdhip_dtype_size(int dtype) { return dtype_size(dtype); }
+
+int hvdhip_get_device(int* device) {
+  if (!device) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "device is NULL");
+  HVDHIP_CHECK(hipGetDevice(device));
+  return ok();
+}
+
+int hvdhip_set_device(int device) {
+  HVDHIP_CHECK(hipSetDevice(device));
+  return ok();
+}
+
+int hvdhip_stream_create(void** stream) {
+  if (!stream) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "stream is NULL");
+  hipStream_t s;
+  HVDHIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *stream = s;
+  return ok();
+}
+
+int hvdhip_stream_destroy(void* stream) {
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int dev = 0;
+  HVDHIP_CHECK(hipGetDevice(&dev));
+  {
+    // Drop the stream's idle events with it.
+    EventPools& p = pools();
+    std::lock_guard<std::mutex> g(p.mu);
+    auto key = std::make_pair(dev, s);
+    auto it = p.idle.find(key);
+    if (it != p.idle.end()) {
+      for (hipEvent_t ev : it->second) (void)hipEventDestroy(ev);
+      p.idle.erase(it);
+    }
+    p.filled.erase(key);
+  }
+  HVDHIP_CHECK(hipStreamDestroy(s));
+  return ok();
+}
+
+int hvdhip_stream_synchronize(void* stream) {
+  HVDHIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  return ok();
+}
+
+int hvdhip_stream_wait_event(void* stream, void* event) {
+  if (!event) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "event is NULL");
+  HVDHIP_CHECK(hipStreamWaitEvent(static_cast<hipStream_t>(stream), static_cast<hipEvent_t>(event), 0));
+  return ok();
+}
+
+int hvdhip_event_acquire(void* stream, void** event) {
+  if (!event) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "event is NULL");
+  int dev = 0;
+  HVDHIP_CHECK(hipGetDevice(&dev));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  EventPools& p = pools();
+  {
+    std::lock_guard<std::mutex> g(p.mu);
+    auto key = std::make_pair(dev, s);
+    auto& q = p.idle[key];
+    if (!p.filled[key]) {
+      for (int i = 0; i < kPrepopulate; ++i) {
+        hipEvent_t ev;
+        HVDHIP_CHECK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+        q.push_back(ev);
+      }
+      p.filled[key] = true;
+    }
+    if (!q.empty()) {
+      *event = q.back();
+      q.pop_back();
+      return ok();
+    }
+  }
+  hipEvent_t ev;
+  HVDHIP_CHECK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+  *event = ev;
+  return ok();
+}
+
+int hvdhip_event_record(void* event, void* stream) {
+  if (!event) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "event is NULL");
+  HVDHIP_CHECK(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
+  return ok();
+}
+
+int hvdhip_event_query(void* event, int* done) {
+  if (!event || !done) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "event or done is NULL");
+  hipError_t e = hipEventQuery(static_cast<hipEvent_t>(event));
+  if (e == hipSuccess) {
+    *done = 1;
+    return ok();
+  }
+  if (e == hipErrorNotReady) {
+    *done = 0;
+    return ok();
+  }
+  return fail((int)e, "hipEventQuery failed: %s", hipGetErrorString(e));
+}
+
+int hvdhip_event_synchronize(void* event) {
+  if (!event) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "event is NULL");
+  HVDHIP_CHECK(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+  return ok();
+}
+
+int hvdhip_event_release(void* stream, void* event) {
+  if (!event) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "event is NULL");
+  int dev = 0;
+  HVDHIP_CHECK(hipGetDevice(&dev));
+  EventPools& p = pools();
+  std::lock_guard<std::mutex> g(p.mu);
+  p.idle[std::make_pair(dev, static_cast<hipStream_t>(stream))].push_back(static_cast<hipEvent_t>(event));
+  return ok();
+}
+
+int hvdhip_event_pool_size(void* stream, int* count) {
+  if (!count) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "count is NULL");
+  int dev = 0;
+  HVDHIP_CHECK(hipGetDevice(&dev));
+  EventPools& p = pools();
+  std::lock_guard<std::mutex> g(p.mu);
+  auto it = p.idle.find(std::make_pair(dev, static_cast<hipStream_t>(stream)));
+  *count = it == p.idle.end() ? 0 : (int)it->second.size();
+  return ok();
+}
+
+int hvdhip_memcpy_async(void* dst, const void* src, size_t count, int kind, void* stream) {
+  hipMemcpyKind k;
+  switch (kind) {
+  case HVDHIP_MEMCPY_H2D: k = hipMemcpyHostToDevice; break;
+  case HVDHIP_MEMCPY_D2H: k = hipMemcpyDeviceToHost; break;
+  case HVDHIP_MEMCPY_D2D: k = hipMemcpyDeviceToDevice; break;
+  default: return fail(HVDHIP_ERR_INVALID_ARGUMENT, "unknown memcpy kind %d", kind);
+  }
+  if (count == 0) return ok();
+  HVDHIP_CHECK(hipMemcpyAsync(dst, src, count, k, static_cast<hipStream_t>(stream)));
+  return ok();
+}
+
+int hvdhip_timer_create(void** timer) {
+  if (!timer) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "timer is NULL");
+  Timer* t = new Timer();
+  hipError_t e = hipEventCreate(&t->start);
+  if (e == hipSuccess) {
+    e = hipEventCreate(&t->stop);
+    if (e != hipSuccess) (void)hipEventDestroy(t->start);
+  }
+  if (e != hipSuccess) {
+    delete t;
+    return fail((int)e, "hipEventCreate failed: %s", hipGetErrorString(e));
+  }
+  *timer = t;
+  return ok();
+}
+
+int hvdhip_timer_start(void* timer, void* stream) {
+  if (!timer) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "timer is NULL");
+  HVDHIP_CHECK(hipEventRecord(static_cast<Timer*>(timer)->start, static_cast<hipStream_t>(stream)));
+  return ok();
+}
+
+int hvdhip_timer_stop(void* timer, void* stream) {
+  if (!timer) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "timer is NULL");
+  HVDHIP_CHECK(hipEventRecord(static_cast<Timer*>(timer)->stop, static_cast<hipStream_t>(stream)));
+  return ok();
+}
+
+int hvdhip_timer_elapsed_ms(void* timer, float* ms) {
+  if (!timer || !ms) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "timer or ms is NULL");
+  Timer* t = static_cast<Timer*>(timer);
+  HVDHIP_CHECK(hipEventSynchronize(t->stop));
+  HVDHIP_CHECK(hipEventElapsedTime(ms, t->start, t->stop));
+  return ok();
+}
+
+int hvdhip_timer_destroy(void* timer) {
+  if (!timer) return ok();
+  Timer* t = static_cast<Timer*>(timer);
+  (void)hipEventDestroy(t->start);
+  (void)hipEventDestroy(t->stop);
+  delete t;
+  return ok();
+}
+
+}  // extern "C"

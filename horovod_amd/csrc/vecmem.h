@@ -1,0 +1,69 @@
+// vecmem.h -- lane-level vector access to global memory (device code).
+//
+// A lane moves N elements of T as one 16- or 8-byte instruction whose address
+// needs only the alignment of a single T: gfx950 serves multi-dword global
+// accesses at any alignment, so callers need no alignment ladder and no head
+// peeling, and naturally aligned data costs nothing extra.
+#ifndef HVDHIP_VECMEM_H
+#define HVDHIP_VECMEM_H
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace hvdhip {
+
+typedef _Float16 half_t;
+
+// Pointer into global (device) memory.  Addresses that arrive as integers
+// from a table would otherwise be generic pointers and use flat instructions.
+template <typename T>
+using gptr = __attribute__((address_space(1))) T*;
+
+template <typename T>
+__device__ __forceinline__ gptr<T> as_global(uint64_t addr) {
+  return reinterpret_cast<gptr<T>>(addr);
+}
+template <typename T>
+__device__ __forceinline__ gptr<T> as_global(T* p) {
+  return reinterpret_cast<gptr<T>>(reinterpret_cast<uint64_t>(p));
+}
+
+template <int BYTES>
+struct RawSel;
+template <>
+struct RawSel<16> {
+  typedef uint32_t type __attribute__((ext_vector_type(4)));
+};
+template <>
+struct RawSel<8> {
+  typedef uint32_t type __attribute__((ext_vector_type(2)));
+};
+// The same register type, declared with the alignment of one element.
+template <int BYTES, int ALIGN>
+struct Raw {
+  typedef typename RawSel<BYTES>::type type __attribute__((aligned(ALIGN)));
+};
+
+// N elements of T held in registers.
+template <typename T, int N>
+struct Arr {
+  T v[N];
+};
+
+template <typename T, int N>
+__device__ __forceinline__ Arr<T, N> ldv(gptr<const T> p) {
+  typedef typename Raw<(int)sizeof(T) * N, (int)alignof(T)>::type R;
+  const typename RawSel<(int)sizeof(T) * N>::type r = *reinterpret_cast<gptr<const R>>(p);
+  return __builtin_bit_cast(Arr<T, N>, r);
+}
+
+template <typename T, int N>
+__device__ __forceinline__ void stv(gptr<T> p, const Arr<T, N>& a) {
+  typedef typename Raw<(int)sizeof(T) * N, (int)alignof(T)>::type R;
+  *reinterpret_cast<gptr<R>>(p) = __builtin_bit_cast(typename RawSel<(int)sizeof(T) * N>::type, a);
+}
+
+}  // namespace hvdhip
+
+#endif  // HVDHIP_VECMEM_H

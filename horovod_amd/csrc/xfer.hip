@@ -1,0 +1,509 @@
+// xfer.hip -- batched fusion-buffer packing and unpacking, with the pre/post
+// scale and the fp32<->fp16 compression cast fused in, plus the whole-buffer
+// scale.  gfx950 only.
+//
+// One launch moves a whole fused response.  The host describes it with two
+// device-resident tables: one segment per tensor (addresses, fusion-buffer
+// offset, element count) and one chunk per workgroup (segment number, chunk
+// number inside the segment).  A workgroup of four wave64 wavefronts streams
+// its chunk with 16-byte accesses per lane, several loads in flight before
+// the first store; consecutive workgroups touch consecutive addresses of a
+// large tensor, so a single big tensor is spread over all XCDs and HBM stacks
+// while a tiny one costs a single short workgroup.  This is bandwidth-bound
+// byte/element work: no LDS and no matrix cores are involved.
+//
+// All vector accesses are declared with element alignment only.  gfx950
+// serves multi-dword global accesses at any alignment, so no alignment
+// ladder or head peeling is needed; 16-byte aligned data (the normal case:
+// fusion offsets are padded to 16 bytes) takes exactly the same instructions.
+//
+// Arithmetic follows the reference's CPU path (ScaleBufferCPUImpl,
+// ops/collective_operations.h:91-127), not its CUDA kernels: fp16 is scaled
+// in fp32 with an fp32 factor and rounded to nearest even once; integers are
+// scaled in double and truncated toward zero.
+#include <algorithm>
+#include <cstring>
+#include <list>
+#include <mutex>
+
+#include "internal.h"
+#include "vecmem.h"
+
+namespace hvdhip {
+namespace {
+
+// ----------------------------------------------------------------------
+// Device side
+// ----------------------------------------------------------------------
+
+// Each Op gives the source and destination element types, the number of
+// elements per lane access (16 bytes on the wider side), the by-value launch
+// parameter and the per-element function.
+
+// Plain copy of elements as unsigned integers of the same width: bit-exact
+// for every dtype.
+template <typename U>
+struct Copy {
+  typedef U S;
+  typedef U D;
+  static constexpr int VEC = 16 / (int)sizeof(U);
+  struct P {};
+  static __device__ __forceinline__ D f(S x, P) { return x; }
+};
+
+// out = (T)(factor * in): factor type TS is double for u8/i8/i32/i64/f64 and
+// float for f32 (ops/collective_operations.cc:119-140).
+template <typename T, typename TS>
+struct Scale {
+  typedef T S;
+  typedef T D;
+  static constexpr int VEC = 16 / (int)sizeof(T);
+  struct P {
+    TS s;
+  };
+  static __device__ __forceinline__ D f(S x, P p) { return (T)(p.s * x); }
+};
+
+// fp16 scaled through fp32 with an fp32 factor, one rounding to nearest even
+// (ops/collective_operations.h:99-127).
+struct ScaleHalf {
+  typedef half_t S;
+  typedef half_t D;
+  static constexpr int VEC = 8;
+  struct P {
+    float s;
+  };
+  static __device__ __forceinline__ D f(S x, P p) { return (half_t)(p.s * (float)x); }
+};
+
+// fp32 -> fp16 with the prescale applied in fp32 first: a single rounding.
+struct PackF32F16 {
+  typedef float S;
+  typedef half_t D;
+  static constexpr int VEC = 4;
+  struct P {
+    float s;
+  };
+  static __device__ __forceinline__ D f(S x, P p) { return (half_t)(p.s * x); }
+};
+
+// fp32 -> fp16 first (horovod/torch/compression.py:49-55), then the fp16
+// scale: two roundings, the order of the reference pipeline.
+struct PackF32F16CastFirst {
+  typedef float S;
+  typedef half_t D;
+  static constexpr int VEC = 4;
+  struct P {
+    float s;
+  };
+  static __device__ __forceinline__ D f(S x, P p) {
+    half_t h = (half_t)x;
+    return (half_t)(p.s * (float)h);
+  }
+};
+
+// Postscale on the fp16 value (rounded back to fp16), then the exact widening
+// of Compression.fp16.decompress (horovod/torch/compression.py:58-64).
+struct UnpackF16F32 {
+  typedef half_t S;
+  typedef float D;
+  static constexpr int VEC = 4;
+  struct P {
+    float s;
+  };
+  static __device__ __forceinline__ D f(S x, P p) {
+    half_t h = (half_t)(p.s * (float)x);
+    return (float)h;
+  }
+};
+
+constexpr int kUnroll = 4;
+
+// Streams n elements from src to dst through Op::f with the whole workgroup.
+template <class Op>
+__device__ __forceinline__ void stream_range(gptr<const typename Op::S> src,
+                                             gptr<typename Op::D> dst, uint32_t n,
+                                             typename Op::P p) {
+  typedef typename Op::S S;
+  typedef typename Op::D D;
+  constexpr int VEC = Op::VEC;
+  // src and dst may be the same buffer (in-place scale): every lane loads all
+  // of an iteration's vectors before it stores any, and touches no address
+  // another lane touches.
+  const uint32_t nv = n / VEC;
+  uint32_t v = threadIdx.x;
+  for (; v + (kUnroll - 1) * kWG < nv; v += kUnroll * kWG) {
+    Arr<S, VEC> x[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) x[u] = ldv<S, VEC>(src + (size_t)(v + u * kWG) * VEC);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      Arr<D, VEC> y;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) y.v[j] = Op::f(x[u].v[j], p);
+      stv<D, VEC>(dst + (size_t)(v + u * kWG) * VEC, y);
+    }
+  }
+  for (; v < nv; v += kWG) {
+    const Arr<S, VEC> x = ldv<S, VEC>(src + (size_t)v * VEC);
+    Arr<D, VEC> y;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) y.v[j] = Op::f(x.v[j], p);
+    stv<D, VEC>(dst + (size_t)v * VEC, y);
+  }
+  const uint32_t t = nv * VEC + threadIdx.x;  // fewer than VEC elements remain
+  if (t < n) dst[t] = Op::f(src[t], p);
+}
+
+enum Mode { kPack = 0, kUnpack = 1, kDirect = 2 };
+
+// One workgroup per chunk-table entry.
+//   kPack:   src = seg.tensor,        dst = base + seg.off (pad bytes zeroed)
+//   kUnpack: src = base + seg.off,    dst = seg.output
+//   kDirect: src = seg.tensor,        dst = seg.output
+template <class Op, int MODE>
+__global__ __launch_bounds__(kWG) void xfer_k(const Seg* __restrict__ segs,
+                                              const Chunk* __restrict__ chunks, uint64_t base,
+                                              uint32_t chunk_units, typename Op::P p) {
+  typedef typename Op::S S;
+  typedef typename Op::D D;
+  const Chunk c = chunks[blockIdx.x];
+  const Seg s = segs[c.seg];
+  const uint64_t start = (uint64_t)c.idx * chunk_units;
+  const uint64_t left = s.n - start;
+  const uint32_t n = left < chunk_units ? (uint32_t)left : chunk_units;
+  const uint64_t src_addr = (MODE == kUnpack) ? base + s.off : s.tensor;
+  const uint64_t dst_addr = (MODE == kPack) ? base + s.off : s.output;
+  gptr<const S> src = as_global<const S>(src_addr) + start;
+  gptr<D> dst = as_global<D>(dst_addr) + start;
+  stream_range<Op>(src, dst, n, p);
+  if (MODE == kPack && left <= chunk_units) {
+    // Last chunk of the tensor: zero the bytes up to the next 16-byte boundary.
+    const uint64_t nbytes = s.n * sizeof(D);
+    const uint32_t pad = (uint32_t)((16 - (nbytes & 15)) & 15);
+    if (threadIdx.x < pad) as_global<uint8_t>(dst_addr)[nbytes + threadIdx.x] = 0;
+  }
+}
+
+// Contiguous buffer: workgroup b handles elements [b*tile, (b+1)*tile).
+template <class Op>
+__global__ __launch_bounds__(kWG) void contig_k(const typename Op::S* src,
+                                                typename Op::D* dst, uint64_t n,
+                                                uint32_t tile, typename Op::P p) {
+  const uint64_t start = (uint64_t)blockIdx.x * tile;
+  const uint64_t left = n - start;
+  const uint32_t m = left < tile ? (uint32_t)left : tile;
+  stream_range<Op>(as_global(src + start), as_global(dst + start), m, p);
+}
+
+// ----------------------------------------------------------------------
+// Host side
+// ----------------------------------------------------------------------
+
+template <class Op, int MODE>
+int launch_xfer(const DevTables& t, uint64_t base, typename Op::P p, hipStream_t stream) {
+  if (t.nchunks == 0) return 0;
+  hipLaunchKernelGGL((xfer_k<Op, MODE>), dim3(t.nchunks), dim3(kWG), 0, stream, t.segs, t.chunks,
+                     base, t.chunk_units, p);
+  HVDHIP_CHECK_LAUNCH("xfer_k");
+  return 0;
+}
+
+// Dispatches the same-dtype transfer over MODE; the tables count elements of
+// dtype.  scale == 1.0 is a plain copy, valid for every dtype.
+template <int MODE>
+int launch_same_dtype(const DevTables& t, uint64_t base, double scale, int dtype,
+                      hipStream_t stream) {
+  if (scale == 1.0) {
+    switch (dtype_size(dtype)) {
+    case 1: return launch_xfer<Copy<uint8_t>, MODE>(t, base, {}, stream);
+    case 2: return launch_xfer<Copy<uint16_t>, MODE>(t, base, {}, stream);
+    case 4: return launch_xfer<Copy<uint32_t>, MODE>(t, base, {}, stream);
+    case 8: return launch_xfer<Copy<uint64_t>, MODE>(t, base, {}, stream);
+    default: return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE, "unknown dtype %d", dtype);
+    }
+  }
+  switch (dtype) {
+  case HVDHIP_UINT8: return launch_xfer<Scale<uint8_t, double>, MODE>(t, base, {scale}, stream);
+  case HVDHIP_INT8: return launch_xfer<Scale<int8_t, double>, MODE>(t, base, {scale}, stream);
+  case HVDHIP_INT32: return launch_xfer<Scale<int32_t, double>, MODE>(t, base, {scale}, stream);
+  case HVDHIP_INT64: return launch_xfer<Scale<int64_t, double>, MODE>(t, base, {scale}, stream);
+  case HVDHIP_FLOAT16: return launch_xfer<ScaleHalf, MODE>(t, base, {(float)scale}, stream);
+  case HVDHIP_FLOAT32: return launch_xfer<Scale<float, float>, MODE>(t, base, {(float)scale}, stream);
+  case HVDHIP_FLOAT64: return launch_xfer<Scale<double, double>, MODE>(t, base, {scale}, stream);
+  default:
+    return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE, "dtype %d cannot be scaled by a factor other than 1", dtype);
+  }
+}
+
+bool scalable(int dtype) {
+  switch (dtype) {
+  case HVDHIP_UINT8: case HVDHIP_INT8: case HVDHIP_INT32: case HVDHIP_INT64:
+  case HVDHIP_FLOAT16: case HVDHIP_FLOAT32: case HVDHIP_FLOAT64: return true;
+  default: return false;
+  }
+}
+
+template <class Op>
+int launch_contig(const void* in, void* out, int64_t n, typename Op::P p, hipStream_t stream) {
+  const uint32_t tile = chunk_bytes() / (uint32_t)std::max(sizeof(typename Op::S), sizeof(typename Op::D));
+  const uint64_t blocks = ((uint64_t)n + tile - 1) / tile;
+  if (blocks > 0x7fffffffull) return fail(HVDHIP_ERR_TOO_LARGE, "buffer of %lld elements is too large", (long long)n);
+  hipLaunchKernelGGL((contig_k<Op>), dim3((uint32_t)blocks), dim3(kWG), 0, stream,
+                     static_cast<const typename Op::S*>(in), static_cast<typename Op::D*>(out),
+                     (uint64_t)n, tile, p);
+  HVDHIP_CHECK_LAUNCH("contig_k");
+  return 0;
+}
+
+// ---- cache of tables for the array-taking entry points ----------------
+
+struct CachedCopy {
+  std::vector<uint64_t> key;  // unit size, n, then out/in/size triples
+  DevTables tables;
+};
+
+struct CopyCache {
+  std::mutex mu;
+  std::list<CachedCopy> lru;  // front = most recent
+};
+CopyCache& copy_cache() {
+  static CopyCache* c = new CopyCache();
+  return *c;
+}
+constexpr size_t kCopyCacheCapacity = 64;
+
+// Finds or builds the tables for (out, in, sizes) with elements of unit bytes.
+int cached_tables(void* const* out, const void* const* in, const size_t* sizes, int n,
+                  uint32_t unit, DevTables* result) {
+  std::vector<uint64_t> key;
+  key.reserve(2 + 3 * (size_t)n);
+  key.push_back(unit);
+  key.push_back((uint64_t)n);
+  for (int i = 0; i < n; ++i) {
+    key.push_back((uint64_t)(uintptr_t)out[i]);
+    key.push_back((uint64_t)(uintptr_t)in[i]);
+    key.push_back((uint64_t)sizes[i]);
+  }
+  CopyCache& c = copy_cache();
+  std::lock_guard<std::mutex> g(c.mu);
+  for (auto it = c.lru.begin(); it != c.lru.end(); ++it) {
+    if (it->key == key) {
+      c.lru.splice(c.lru.begin(), c.lru, it);
+      *result = c.lru.front().tables;
+      return 0;
+    }
+  }
+  std::vector<Seg> segs((size_t)n);
+  for (int i = 0; i < n; ++i)
+    segs[i] = Seg{(uint64_t)(uintptr_t)in[i], (uint64_t)(uintptr_t)out[i], 0, sizes[i] / unit};
+  CachedCopy entry;
+  entry.key.swap(key);
+  int rc = build_tables(segs, chunk_bytes() / unit, &entry.tables);
+  if (rc) return rc;
+  if (c.lru.size() >= kCopyCacheCapacity) {
+    // Tables may still be read by queued kernels: wait before freeing.
+    HVDHIP_CHECK(hipDeviceSynchronize());
+    free_tables(&c.lru.back().tables);
+    c.lru.pop_back();
+  }
+  c.lru.push_front(std::move(entry));
+  *result = c.lru.front().tables;
+  return 0;
+}
+
+int check_arrays(void* const* out, const void* const* in, const size_t* sizes, int n) {
+  if (n < 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "num_copies is negative");
+  if (n > 0 && (!out || !in || !sizes)) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "out, in or sizes is NULL");
+  for (int i = 0; i < n; ++i)
+    if (sizes[i] && (!out[i] || !in[i]))
+      return fail(HVDHIP_ERR_INVALID_ARGUMENT, "copy %d has a NULL pointer with non-zero size", i);
+  return 0;
+}
+
+}  // namespace
+}  // namespace hvdhip
+
+using namespace hvdhip;
+
+struct hvdhip_fusion_plan {
+  int n = 0;
+  int tensor_dtype = 0;
+  int buffer_dtype = 0;
+  int64_t buffer_len = 0;
+  std::vector<int64_t> offsets;
+  DevTables tables;
+};
+
+extern "C" {
+
+int hvdhip_batched_d2d_memcpy(void* const* out, const void* const* in, const size_t* sizes,
+                              int num_copies, void* stream) {
+  int rc = check_arrays(out, in, sizes, num_copies);
+  if (rc) return rc;
+  if (num_copies == 0) return ok();
+  DevTables t;
+  rc = cached_tables(out, in, sizes, num_copies, 1, &t);
+  if (rc) return rc;
+  rc = launch_xfer<Copy<uint8_t>, kDirect>(t, 0, {}, static_cast<hipStream_t>(stream));
+  return rc ? rc : ok();
+}
+
+int hvdhip_batched_scaled_d2d_memcpy(void* const* out, const void* const* in,
+                                     const size_t* sizes, int num_copies, double scale_factor,
+                                     int dtype, void* stream) {
+  int rc = check_arrays(out, in, sizes, num_copies);
+  if (rc) return rc;
+  if (!scalable(dtype))
+    return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported by the scaled batched copy", dtype);
+  if (num_copies == 0) return ok();
+  const uint32_t es = (uint32_t)dtype_size(dtype);
+  for (int i = 0; i < num_copies; ++i) {
+    if (sizes[i] % es)
+      return fail(HVDHIP_ERR_INVALID_ARGUMENT, "size of copy %d is not a multiple of the element size", i);
+    if (((uintptr_t)out[i] | (uintptr_t)in[i]) % es)
+      return fail(HVDHIP_ERR_INVALID_ARGUMENT, "copy %d is not aligned to its element size", i);
+  }
+  DevTables t;
+  rc = cached_tables(out, in, sizes, num_copies, es, &t);
+  if (rc) return rc;
+  rc = launch_same_dtype<kDirect>(t, 0, scale_factor, dtype, static_cast<hipStream_t>(stream));
+  return rc ? rc : ok();
+}
+
+int hvdhip_scale_buffer(const void* fused_input_data, void* buffer_data, int64_t num_elements,
+                        double scale_factor, int dtype, void* stream) {
+  if (!scalable(dtype))
+    return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported by ScaleBuffer", dtype);
+  if (num_elements < 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "num_elements is negative");
+  if (num_elements == 0) return ok();
+  if (!fused_input_data || !buffer_data) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "buffer is NULL");
+  if (((uintptr_t)fused_input_data | (uintptr_t)buffer_data) % (uintptr_t)dtype_size(dtype))
+    return fail(HVDHIP_ERR_INVALID_ARGUMENT, "buffer is not aligned to its element size");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const void* in = fused_input_data;
+  void* out = buffer_data;
+  const int64_t n = num_elements;
+  int rc;
+  switch (dtype) {
+  case HVDHIP_UINT8: rc = launch_contig<Scale<uint8_t, double>>(in, out, n, {scale_factor}, s); break;
+  case HVDHIP_INT8: rc = launch_contig<Scale<int8_t, double>>(in, out, n, {scale_factor}, s); break;
+  case HVDHIP_INT32: rc = launch_contig<Scale<int32_t, double>>(in, out, n, {scale_factor}, s); break;
+  case HVDHIP_INT64: rc = launch_contig<Scale<int64_t, double>>(in, out, n, {scale_factor}, s); break;
+  case HVDHIP_FLOAT16: rc = launch_contig<ScaleHalf>(in, out, n, {(float)scale_factor}, s); break;
+  case HVDHIP_FLOAT32: rc = launch_contig<Scale<float, float>>(in, out, n, {(float)scale_factor}, s); break;
+  default: rc = launch_contig<Scale<double, double>>(in, out, n, {scale_factor}, s); break;
+  }
+  return rc ? rc : ok();
+}
+
+int hvdhip_fusion_plan_create(const void* const* tensors, void* const* outputs,
+                              const int64_t* num_elements, int n, int tensor_dtype,
+                              int buffer_dtype, hvdhip_fusion_plan** plan) {
+  if (!plan) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "plan is NULL");
+  *plan = nullptr;
+  if (n < 0 || (n > 0 && (!tensors || !outputs || !num_elements)))
+    return fail(HVDHIP_ERR_INVALID_ARGUMENT, "bad entry arrays");
+  const int64_t ts = dtype_size(tensor_dtype);
+  const int64_t bs = dtype_size(buffer_dtype);
+  if (ts < 0 || bs < 0) return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE, "unknown dtype");
+  if (buffer_dtype != tensor_dtype &&
+      !(tensor_dtype == HVDHIP_FLOAT32 && buffer_dtype == HVDHIP_FLOAT16))
+    return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE,
+                "buffer dtype %d with tensor dtype %d: only FLOAT32 tensors in a FLOAT16 buffer convert",
+                buffer_dtype, tensor_dtype);
+  std::vector<Seg> segs((size_t)n);
+  std::vector<int64_t> offsets((size_t)n);
+  int64_t off = 0;
+  for (int i = 0; i < n; ++i) {
+    if (num_elements[i] < 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "entry %d has a negative size", i);
+    if (num_elements[i] > 0) {
+      if (!tensors[i] || !outputs[i]) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "entry %d has a NULL pointer", i);
+      if (((uintptr_t)tensors[i] | (uintptr_t)outputs[i]) % (uintptr_t)ts)
+        return fail(HVDHIP_ERR_INVALID_ARGUMENT, "entry %d is not aligned to its element size", i);
+    }
+    offsets[i] = off;
+    segs[i] = Seg{(uint64_t)(uintptr_t)tensors[i], (uint64_t)(uintptr_t)outputs[i], (uint64_t)off,
+                  (uint64_t)num_elements[i]};
+    off += 16 * ((num_elements[i] * bs + 15) / 16);  // ops/gpu_operations.cc:141
+  }
+  hvdhip_fusion_plan* p = new hvdhip_fusion_plan();
+  p->n = n;
+  p->tensor_dtype = tensor_dtype;
+  p->buffer_dtype = buffer_dtype;
+  p->buffer_len = off;
+  p->offsets.swap(offsets);
+  int rc = build_tables(segs, chunk_bytes() / (uint32_t)std::max(ts, bs), &p->tables);
+  if (rc) {
+    delete p;
+    return rc;
+  }
+  *plan = p;
+  return ok();
+}
+
+int hvdhip_fusion_plan_destroy(hvdhip_fusion_plan* plan) {
+  if (!plan) return ok();
+  // Queued kernels may still read the tables.
+  HVDHIP_CHECK(hipDeviceSynchronize());
+  int rc = free_tables(&plan->tables);
+  delete plan;
+  return rc ? rc : ok();
+}
+
+int64_t hvdhip_fusion_plan_buffer_len(const hvdhip_fusion_plan* plan) {
+  return plan ? plan->buffer_len : -1;
+}
+
+int hvdhip_fusion_plan_offsets(const hvdhip_fusion_plan* plan, int64_t* offsets) {
+  if (!plan || (plan->n > 0 && !offsets)) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "plan or offsets is NULL");
+  for (int i = 0; i < plan->n; ++i) offsets[i] = plan->offsets[(size_t)i];
+  return ok();
+}
+
+int64_t hvdhip_fusion_plan_num_chunks(const hvdhip_fusion_plan* plan) {
+  return plan ? (int64_t)plan->tables.nchunks : -1;
+}
+
+int hvdhip_fusion_pack(hvdhip_fusion_plan* plan, void* fusion_buffer, double scale_factor,
+                       unsigned flags, void* stream) {
+  if (!plan) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "plan is NULL");
+  if (plan->buffer_len > 0 && !fusion_buffer) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "fusion_buffer is NULL");
+  if ((uintptr_t)fusion_buffer % 16) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "fusion_buffer must be 16-byte aligned");
+  if (flags & ~HVDHIP_PACK_CAST_THEN_SCALE) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "unknown flags 0x%x", flags);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uint64_t base = (uint64_t)(uintptr_t)fusion_buffer;
+  int rc;
+  if (plan->buffer_dtype != plan->tensor_dtype) {
+    if (flags & HVDHIP_PACK_CAST_THEN_SCALE)
+      rc = launch_xfer<PackF32F16CastFirst, kPack>(plan->tables, base, {(float)scale_factor}, s);
+    else
+      rc = launch_xfer<PackF32F16, kPack>(plan->tables, base, {(float)scale_factor}, s);
+  } else {
+    if (flags) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "HVDHIP_PACK_CAST_THEN_SCALE needs a converting plan");
+    if (scale_factor != 1.0 && !scalable(plan->tensor_dtype))
+      return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE, "dtype %d cannot be scaled", plan->tensor_dtype);
+    rc = launch_same_dtype<kPack>(plan->tables, base, scale_factor, plan->tensor_dtype, s);
+  }
+  return rc ? rc : ok();
+}
+
+int hvdhip_fusion_unpack(hvdhip_fusion_plan* plan, const void* fusion_buffer,
+                         double scale_factor, void* stream) {
+  if (!plan) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "plan is NULL");
+  if (plan->buffer_len > 0 && !fusion_buffer) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "fusion_buffer is NULL");
+  if ((uintptr_t)fusion_buffer % 16) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "fusion_buffer must be 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uint64_t base = (uint64_t)(uintptr_t)fusion_buffer;
+  int rc;
+  if (plan->buffer_dtype != plan->tensor_dtype) {
+    rc = launch_xfer<UnpackF16F32, kUnpack>(plan->tables, base, {(float)scale_factor}, s);
+  } else {
+    if (scale_factor != 1.0 && !scalable(plan->tensor_dtype))
+      return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE, "dtype %d cannot be scaled", plan->tensor_dtype);
+    rc = launch_same_dtype<kUnpack>(plan->tables, base, scale_factor, plan->tensor_dtype, s);
+  }
+  return rc ? rc : ok();
+}
+
+}  // extern "C"

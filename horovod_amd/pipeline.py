@@ -1,0 +1,126 @@
+"""The allreduce op sequence of the reference on one GPU, driven through the C ABI.
+
+Mirrors NCCLAllreduce::Execute (ops/nccl_operations.cc:156-214) for a list of
+gradient tensors: the tensors are grouped into fusion cycles by the greedy
+planner, and every cycle runs
+
+    fused (more than one entry):  scaled pack -> sum with the peer chunk(s) -> scaled unpack
+    single entry:                 prescale tensor -> output (out of place), sum in place, postscale
+
+with the inter-GPU collective replaced by the local reduce-sum against peer
+buffers resident on the same device.  Cycles alternate over `num_streams`
+streams, each with its own fusion buffer, as the reference rotates
+current_nccl_stream after every op (ops/gpu_operations.cc:101-103).
+
+This module only sequences calls; all arithmetic happens in libhvdhip.so.
+"""
+import torch
+
+from . import host as H
+from ._lib import DTYPE, dtype_size
+from .workloads import FUSION_THRESHOLD, fuse
+
+
+class Cycle:
+    def __init__(self, indices, plan, single):
+        self.indices = indices
+        self.plan = plan          # FusionPlan, or None for a single-entry response
+        self.single = single      # (tensor_ptr, output_ptr, count) for a single-entry response
+        self.buffer_elems = 0     # elements of the fusion buffer (padded) or of the single tensor
+        self.payload_in = 0       # bytes read from tensors
+        self.payload_buf = 0      # payload bytes in the buffer dtype
+        self.payload_out = 0      # bytes written to outputs
+
+
+class AllreducePipeline:
+    """tensor_ptrs/output_ptrs/counts describe the gradients (device addresses).
+
+    peers: list of callables or None; peer_ptr(cycle_index, peer) must return the
+    device address of that peer's chunk for the cycle, `reduce_fraction` of the
+    cycle's buffer long (1.0 = the whole buffer, 1/8 = one GPU's reduce-scatter
+    share)."""
+
+    def __init__(self, tensor_ptrs, output_ptrs, counts, tensor_dtype, buffer_dtype=None,
+                 threshold=FUSION_THRESHOLD, num_streams=1):
+        self.tensor_dtype = int(tensor_dtype)
+        self.buffer_dtype = int(tensor_dtype if buffer_dtype is None else buffer_dtype)
+        ts, bs = dtype_size(self.tensor_dtype), dtype_size(self.buffer_dtype)
+        self.bs = bs
+        groups = fuse([c * bs for c in counts], threshold)
+        self.cycles = []
+        max_len = 0
+        for g in groups:
+            if len(g) > 1 or self.buffer_dtype != self.tensor_dtype:
+                plan = H.FusionPlan([tensor_ptrs[i] for i in g], [output_ptrs[i] for i in g],
+                                    [counts[i] for i in g], self.tensor_dtype, self.buffer_dtype)
+                cyc = Cycle(g, plan, None)
+                cyc.buffer_elems = plan.buffer_len // bs
+                max_len = max(max_len, plan.buffer_len)
+            else:
+                i = g[0]
+                cyc = Cycle(g, None, (tensor_ptrs[i], output_ptrs[i], counts[i]))
+                cyc.buffer_elems = counts[i]
+            n = sum(counts[i] for i in g)
+            cyc.payload_in, cyc.payload_buf, cyc.payload_out = n * ts, n * bs, n * ts
+            self.cycles.append(cyc)
+        self.streams = [H.Stream() for _ in range(num_streams)]
+        self.buffers = [torch.empty(max(max_len, 16), dtype=torch.uint8, device="cuda") for _ in range(num_streams)]
+        torch.cuda.synchronize()
+
+    def reduce_elems(self, cyc, fraction):
+        n = int(cyc.buffer_elems * fraction)
+        return max(n - n % 8, 0) if fraction < 1.0 else cyc.buffer_elems
+
+    def run(self, prescale, postscale, peer_ptr=None, num_peers=0, fraction=1.0, kway=True, flags=0):
+        """Queues every cycle; returns without synchronising."""
+        for ci, cyc in enumerate(self.cycles):
+            slot = ci % len(self.streams)
+            s = self.streams[slot]
+            if cyc.plan is not None:
+                fb = self.buffers[slot].data_ptr()
+                cyc.plan.pack(fb, prescale, s, flags)
+                res = fb
+            else:
+                t, o, n = cyc.single
+                if prescale != 1.0:
+                    H.scale_buffer(t, o, n, prescale, self.tensor_dtype, s)
+                elif t != o:
+                    H.batched_d2d_memcpy([o], [t], [n * self.bs], s)
+                res = o
+            if num_peers:
+                n = self.reduce_elems(cyc, fraction)
+                ptrs = [peer_ptr(ci, p) for p in range(num_peers)]
+                if kway:
+                    H.reduce_sum_k(res, ptrs, n, self.buffer_dtype, s)
+                else:
+                    for p in ptrs:
+                        H.reduce_sum(res, p, n, self.buffer_dtype, s)
+            if cyc.plan is not None:
+                cyc.plan.unpack(self.buffers[slot].data_ptr(), postscale, s)
+            elif postscale != 1.0:
+                t, o, n = cyc.single
+                H.scale_buffer(o, o, n, postscale, self.tensor_dtype, s)
+
+    def synchronize(self):
+        for s in self.streams:
+            s.synchronize()
+
+    def algorithmic_bytes(self, num_peers=0, fraction=1.0, kway=True):
+        """pack = P_in + P_buf, unpack = P_buf + P_out, reduce = (k+2)*C k-way or 3*C per peer."""
+        total = 0
+        for cyc in self.cycles:
+            if cyc.plan is not None:
+                total += cyc.payload_in + cyc.payload_buf + cyc.payload_buf + cyc.payload_out
+            else:
+                total += cyc.payload_in + cyc.payload_out  # prescale tensor -> output
+            if num_peers:
+                c = self.reduce_elems(cyc, fraction) * self.bs
+                total += (num_peers + 2) * c if kway else 3 * c * num_peers
+        return total
+
+    def destroy(self):
+        for cyc in self.cycles:
+            if cyc.plan is not None:
+                cyc.plan.destroy()
+        for s in self.streams:
+            s.destroy()

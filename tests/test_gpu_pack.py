@@ -1,0 +1,251 @@
+"""Parity of the HIP pack / unpack / batched-copy path with the CPU oracle,
+through the C ABI.  Bit-exact for copies; scaled values compared bit-for-bit
+with the oracle's ScaleBuffer on the same seeded inputs."""
+import numpy as np
+import pytest
+
+from oracle_util import F16, F32, F64, I8, I32, I64, U8, U16, NP_OF, SIZE_OF
+
+pytestmark = pytest.mark.gpu
+
+from gpu_util import Arena  # noqa: E402
+
+EDGE_BYTES = [0, 1, 2, 3, 15, 16, 17, 31, 32, 33, 255, 256, 257, 4095, 4096, 4097, 32767, 32768, 32769,
+              65536 + 5, 3 * 32768 + 1]
+
+
+def _rand_values(rng, n, dtype):
+    np_t = NP_OF[dtype]
+    if dtype in (F32, F64):
+        return rng.uniform(-1, 1, n).astype(np_t)
+    if dtype == F16:
+        return rng.uniform(-1, 1, n).astype(np.float16)
+    if dtype == I64:
+        return rng.integers(-2 ** 40, 2 ** 40, n, dtype=np.int64)
+    info = np.iinfo(np_t)
+    return rng.integers(info.min, int(info.max) + 1, n, dtype=np.int64).astype(np_t)
+
+
+def _build(gpu, rng, counts, dtype, misalign=None, out_misalign=None):
+    """Places tensors (seeded values) and zeroed outputs in arenas; returns everything a test needs."""
+    es = SIZE_OF[dtype]
+    total = sum(c * es for c in counts) + 512 * (len(counts) + 2)
+    src, dst = Arena(total), Arena(total, fill=0x5A)
+    offs, ooffs, vals = [], [], []
+    for i, c in enumerate(counts):
+        m = 0 if misalign is None else misalign[i % len(misalign)]
+        om = 0 if out_misalign is None else out_misalign[i % len(out_misalign)]
+        o = src.alloc(c * es, misalign=m)
+        oo = dst.alloc(c * es, misalign=om)
+        v = _rand_values(rng, c, dtype)
+        src.host[o:o + c * es] = v.view(np.uint8)
+        offs.append(o)
+        ooffs.append(oo)
+        vals.append(v)
+    src.upload()
+    dst.upload()
+    return src, dst, offs, ooffs, vals
+
+
+def _raw(v):
+    return v.view(np.uint16) if v.dtype == np.float16 else v
+
+
+def _check_round_trip(gpu, orc, counts, dtype, prescale, postscale, misalign=None, out_misalign=None, seed=0):
+    rng = np.random.default_rng(seed)
+    es = SIZE_OF[dtype]
+    src, dst, offs, ooffs, vals = _build(gpu, rng, counts, dtype, misalign, out_misalign)
+    plan = gpu.H.FusionPlan([src.ptr(o) for o in offs], [dst.ptr(o) for o in ooffs], counts, dtype)
+    try:
+        want_offs = orc.padded_offsets([c * es for c in counts])
+        assert plan.buffer_len == want_offs[-1]
+        assert plan.offsets() == list(want_offs[:-1])
+        fb = gpu.empty(plan.buffer_len + 64, fill=0xCD)
+        plan.pack(fb.data_ptr(), prescale, gpu.stream)
+        buf = gpu.download(fb)
+        # per-tensor parity of the buffer contents with the oracle's ScaleBuffer
+        scaled = []
+        for i, (c, v) in enumerate(zip(counts, vals)):
+            w = _raw(v) if prescale == 1.0 else orc.scale_buffer(_raw(v), prescale, dtype)
+            scaled.append(w)
+            got = buf[want_offs[i]:want_offs[i] + c * es]
+            assert np.array_equal(got, w.view(np.uint8)), "pack: tensor %d of %d elements" % (i, c)
+            pad = buf[want_offs[i] + c * es:want_offs[i + 1]]
+            assert np.all(pad == 0), "pad bytes after tensor %d" % i
+        assert np.all(buf[plan.buffer_len:] == 0xCD), "wrote past buffer_len"
+        plan.unpack(fb.data_ptr(), postscale, gpu.stream)
+        gpu.sync()
+        out = dst.download()
+        touched = np.zeros(out.size, bool)
+        for i, (c, w) in enumerate(zip(counts, scaled)):
+            z = w if postscale == 1.0 else orc.scale_buffer(w, postscale, dtype)
+            got = out[ooffs[i]:ooffs[i] + c * es]
+            assert np.array_equal(got, z.view(np.uint8)), "unpack: tensor %d of %d elements" % (i, c)
+            touched[ooffs[i]:ooffs[i] + c * es] = True
+        assert np.all(out[~touched] == 0x5A), "unpack wrote outside the outputs"
+    finally:
+        plan.destroy()
+
+
+@pytest.mark.parametrize("dtype", [U8, I8, U16, I32, I64, F16, F32, F64])
+def test_pack_unpack_copy_edge_sizes(gpu, orc, dtype):
+    es = SIZE_OF[dtype]
+    counts = [b // es for b in EDGE_BYTES]
+    _check_round_trip(gpu, orc, counts, dtype, 1.0, 1.0, seed=1)
+
+
+@pytest.mark.parametrize("dtype", [U8, I8, I32, I64, F16, F32, F64])
+@pytest.mark.parametrize("prescale,postscale", [(0.125, 1.0), (1.0 / 3.0, 2.5), (0.3, 0.999)])
+def test_pack_unpack_scaled_edge_sizes(gpu, orc, dtype, prescale, postscale):
+    es = SIZE_OF[dtype]
+    counts = [b // es for b in EDGE_BYTES]
+    _check_round_trip(gpu, orc, counts, dtype, prescale, postscale, seed=2)
+
+
+@pytest.mark.parametrize("dtype", [U8, F16, F32, F64])
+def test_pack_unpack_every_misalignment(gpu, orc, dtype):
+    # source and output tensors at every element-aligned offset within 16 bytes
+    es = SIZE_OF[dtype]
+    mis = list(range(0, 16, es))
+    counts = [(1000 + 37 * i) // es + 1 for i in range(2 * len(mis))] + [40000 // es + 3]
+    _check_round_trip(gpu, orc, counts, dtype, 1.0, 1.0, misalign=mis, out_misalign=mis[::-1], seed=3)
+    if dtype != U8:
+        _check_round_trip(gpu, orc, counts, dtype, 0.125, 1.0 / 3.0, misalign=mis, out_misalign=mis[::-1], seed=4)
+
+
+def test_more_entries_than_the_reference_batch_capacity(gpu, orc):
+    # 1,000 entries: the reference needs ceil(1000/160) launches (ops/gpu_operations.cc:145)
+    rng = np.random.default_rng(5)
+    counts = [int(x) for x in rng.integers(1, 3000, 1000)]
+    _check_round_trip(gpu, orc, counts, F32, 0.125, 1.0, seed=5)
+
+
+def test_in_place_outputs_alias_tensors(gpu, orc):
+    # allreduce_async_ passes output == tensor (torch/mpi_ops.py:265)
+    rng = np.random.default_rng(6)
+    counts = [1, 1023, 70001, 16]
+    src, _, offs, _, vals = _build(gpu, rng, counts, F32)
+    ptrs = [src.ptr(o) for o in offs]
+    plan = gpu.H.FusionPlan(ptrs, ptrs, counts, F32)
+    try:
+        fb = gpu.empty(plan.buffer_len)
+        plan.pack(fb.data_ptr(), 0.5, gpu.stream)
+        plan.unpack(fb.data_ptr(), 3.0, gpu.stream)
+        gpu.sync()
+        out = src.download()
+        for o, c, v in zip(offs, counts, vals):
+            want = orc.scale_buffer(orc.scale_buffer(v, 0.5, F32), 3.0, F32)
+            assert np.array_equal(out[o:o + 4 * c], want.view(np.uint8))
+    finally:
+        plan.destroy()
+
+
+def test_empty_plan_and_zero_length_entries(gpu, orc):
+    plan = gpu.H.FusionPlan([], [], [], F32)
+    assert plan.buffer_len == 0 and plan.num_chunks == 0
+    plan.pack(0, 0.5, gpu.stream)
+    plan.unpack(0, 0.5, gpu.stream)
+    gpu.sync()
+    plan.destroy()
+    _check_round_trip(gpu, orc, [0, 5, 0, 0, 9, 0], F32, 0.125, 1.0, seed=7)
+
+
+@pytest.mark.parametrize("prescale", [0.125, 1.0, 1.0 / 3.0, 1e-3])
+@pytest.mark.parametrize("flags", [0, 1])
+def test_converting_pack_fp32_to_fp16(gpu, orc, prescale, flags):
+    # values N(0,1e-4): after the prescale most results are subnormal halves
+    rng = np.random.default_rng(8)
+    counts = [b // 4 for b in EDGE_BYTES] + [100003]
+    src = Arena(sum(counts) * 4 + 512 * (len(counts) + 2))
+    dst = Arena(src.capacity, fill=0x5A)
+    offs, ooffs, vals = [], [], []
+    for i, c in enumerate(counts):
+        o, oo = src.alloc(c * 4, misalign=4 * (i % 4)), dst.alloc(c * 4, misalign=4 * ((i + 1) % 4))
+        v = (rng.standard_normal(c) * 1e-4).astype(np.float32)
+        if c > 8:
+            v[:8] = [0.0, -0.0, 65504.0, 65520.0, -1e9, 6.1e-5, 5.96e-8, 2.98e-8]
+        src.host[o:o + 4 * c] = v.view(np.uint8)
+        offs.append(o), ooffs.append(oo), vals.append(v)
+    src.upload(), dst.upload()
+    plan = gpu.H.FusionPlan([src.ptr(o) for o in offs], [dst.ptr(o) for o in ooffs], counts, F32, F16)
+    try:
+        want_offs = orc.padded_offsets([2 * c for c in counts])
+        assert plan.buffer_len == want_offs[-1]
+        fb = gpu.empty(plan.buffer_len + 64, fill=0xCD)
+        plan.pack(fb.data_ptr(), prescale, gpu.stream, flags=flags)
+        buf = gpu.download(fb)
+        halves = []
+        for i, (c, v) in enumerate(zip(counts, vals)):
+            w = orc.scale_cast_f32_to_f16(v, prescale, cast_first=bool(flags))
+            halves.append(w)
+            got = buf[want_offs[i]:want_offs[i] + 2 * c].view(np.uint16)
+            assert np.array_equal(got, w), "tensor %d: %d of %d halves differ" % (i, int((got != w).sum()), c)
+            assert np.all(buf[want_offs[i] + 2 * c:want_offs[i + 1]] == 0)
+        assert np.all(buf[plan.buffer_len:] == 0xCD)
+        for postscale in (1.0, 4.0, 1.0 / 3.0):
+            plan.unpack(fb.data_ptr(), postscale, gpu.stream)
+            gpu.sync()
+            out = dst.download()
+            for i, (c, w) in enumerate(zip(counts, halves)):
+                want = orc.scale_cast_f16_to_f32(w, postscale)
+                got = out[ooffs[i]:ooffs[i] + 4 * c].view(np.uint32)
+                assert np.array_equal(got, want.view(np.uint32)), "unpack tensor %d postscale %r" % (i, postscale)
+    finally:
+        plan.destroy()
+
+
+def test_batched_d2d_memcpy_arbitrary_bytes(gpu, orc):
+    # the byte-granular entry point: any size, any alignment on either side
+    rng = np.random.default_rng(9)
+    sizes = [0, 1, 2, 3, 5, 15, 16, 17, 100, 4097, 32768, 32771, 100001]
+    sizes = sizes + sizes
+    src = Arena(sum(sizes) + 512 * (len(sizes) + 2))
+    dst = Arena(src.capacity, fill=0x5A)
+    so, do = [], []
+    for i, n in enumerate(sizes):
+        so.append(src.alloc(n, misalign=i % 16))
+        do.append(dst.alloc(n, misalign=(7 * i + 3) % 16))
+        src.host[so[-1]:so[-1] + n] = rng.integers(0, 256, n, dtype=np.uint8)
+    src.upload(), dst.upload()
+    for rep in range(2):  # second call hits the table cache
+        gpu.H.batched_d2d_memcpy([dst.ptr(o) for o in do], [src.ptr(o) for o in so], sizes, gpu.stream)
+    gpu.sync()
+    out = dst.download()
+    touched = np.zeros(out.size, bool)
+    for s, d, n in zip(so, do, sizes):
+        assert np.array_equal(out[d:d + n], src.host[s:s + n])
+        touched[d:d + n] = True
+    assert np.all(out[~touched] == 0x5A)
+
+
+@pytest.mark.parametrize("dtype,scale", [(F32, 0.125), (F32, 1.0), (F16, 1.0 / 3.0), (I32, 0.3), (F64, 0.7)])
+def test_batched_scaled_d2d_memcpy(gpu, orc, dtype, scale):
+    rng = np.random.default_rng(10)
+    es = SIZE_OF[dtype]
+    counts = [1, 3, 4, 5, 1000, 8193, 70001]
+    src, dst, offs, ooffs, vals = _build(gpu, rng, counts, dtype, misalign=[0, es], out_misalign=[es, 0])
+    gpu.H.batched_scaled_d2d_memcpy([dst.ptr(o) for o in ooffs], [src.ptr(o) for o in offs],
+                                    [c * es for c in counts], scale, dtype, gpu.stream)
+    gpu.sync()
+    out = dst.download()
+    for o, c, v in zip(ooffs, counts, vals):
+        want = _raw(v) if scale == 1.0 else orc.scale_buffer(_raw(v), scale, dtype)
+        assert np.array_equal(out[o:o + c * es], want.view(np.uint8))
+
+
+def test_rejected_arguments(gpu):
+    import horovod_amd
+    L = horovod_amd.lib()
+    with pytest.raises(horovod_amd.HvdHipError) as e:
+        gpu.H.FusionPlan([1024], [1024], [4], F16, F32)  # only fp32 tensors in an fp16 buffer convert
+    assert e.value.code == -2
+    with pytest.raises(horovod_amd.HvdHipError):
+        gpu.H.FusionPlan([1026], [1024], [4], F32)  # misaligned for its element size
+    t = gpu.empty(64)
+    plan = gpu.H.FusionPlan([t.data_ptr()], [t.data_ptr()], [4], U16)
+    with pytest.raises(horovod_amd.HvdHipError) as e:
+        plan.pack(t.data_ptr(), 0.5, gpu.stream)  # UINT16 cannot be scaled (collective_operations.cc:141-144)
+    assert e.value.code == -2
+    with pytest.raises(horovod_amd.HvdHipError):
+        plan.pack(t.data_ptr() + 8, 1.0, gpu.stream)  # fusion buffer must be 16-byte aligned
+    plan.destroy()
