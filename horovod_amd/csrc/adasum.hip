@@ -175,8 +175,8 @@ struct Axpby {
 template <>
 struct Axpby<half_t> {
   static __device__ __forceinline__ half_t f(double ca, half_t a, double cb, half_t b) {
-    const float t = __fmul_rn((float)ca, (float)a);
-    return (half_t)__fmaf_rn((float)cb, (float)b, t);
+    const float t = opaque(__fmul_rn((float)ca, (float)a));
+    return (half_t)opaque(__fmaf_rn((float)cb, (float)b, t));
   }
 };
 

@@ -23,9 +23,11 @@ int ok();
 #define HVDHIP_CHECK(call)                                                          \
   do {                                                                              \
     hipError_t hvdhip_e_ = (call);                                                  \
-    if (hvdhip_e_ != hipSuccess)                                                    \
+    if (hvdhip_e_ != hipSuccess) {                                                  \
+      (void)hipGetLastError(); /* the code is returned; leave no stale error behind */ \
       return ::hvdhip::fail((int)hvdhip_e_, "%s failed: %s", #call,                 \
                             hipGetErrorString(hvdhip_e_));                          \
+    }                                                                               \
   } while (0)
 
 // Checks the launch that has just been issued.

@@ -25,7 +25,7 @@ struct Add {
 template <>
 struct Add<half_t> {
   static __device__ __forceinline__ half_t f(half_t r, half_t x) {
-    return (half_t)((float)r + (float)x);
+    return (half_t)opaque((float)r + (float)x);
   }
 };
 

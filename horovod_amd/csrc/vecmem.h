@@ -45,6 +45,15 @@ struct Raw {
   typedef typename RawSel<BYTES>::type type __attribute__((aligned(ALIGN)));
 };
 
+// Returns x unchanged but hides where it came from.  Used between an fp32
+// operation and a narrowing to fp16: without it the compiler fuses the pair
+// into one mixed-precision fma with a +0 addend, which turns a -0 product
+// into +0.  No instruction is emitted.
+__device__ __forceinline__ float opaque(float x) {
+  asm("" : "+v"(x));
+  return x;
+}
+
 // N elements of T held in registers.
 template <typename T, int N>
 struct Arr {

@@ -73,7 +73,7 @@ struct ScaleHalf {
   struct P {
     float s;
   };
-  static __device__ __forceinline__ D f(S x, P p) { return (half_t)(p.s * (float)x); }
+  static __device__ __forceinline__ D f(S x, P p) { return (half_t)opaque(p.s * (float)x); }
 };
 
 // fp32 -> fp16 with the prescale applied in fp32 first: a single rounding.
@@ -84,7 +84,7 @@ struct PackF32F16 {
   struct P {
     float s;
   };
-  static __device__ __forceinline__ D f(S x, P p) { return (half_t)(p.s * x); }
+  static __device__ __forceinline__ D f(S x, P p) { return (half_t)opaque(p.s * x); }
 };
 
 // fp32 -> fp16 first (horovod/torch/compression.py:49-55), then the fp16
@@ -98,7 +98,7 @@ struct PackF32F16CastFirst {
   };
   static __device__ __forceinline__ D f(S x, P p) {
     half_t h = (half_t)x;
-    return (half_t)(p.s * (float)h);
+    return (half_t)opaque(p.s * (float)h);
   }
 };
 
@@ -112,7 +112,7 @@ struct UnpackF16F32 {
     float s;
   };
   static __device__ __forceinline__ D f(S x, P p) {
-    half_t h = (half_t)(p.s * (float)x);
+    half_t h = (half_t)opaque(p.s * (float)x);
     return (float)h;
   }
 };
