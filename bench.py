@@ -39,6 +39,11 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--kernel-only", action="store_true",
                     help="only launch the dominant kernel (for rocprofv3 runs)")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="only launch a plain 256 MiB device copy (scales rocprofv3 byte counters)")
+    ap.add_argument("--replicas", type=int, default=8,
+                    help="independent copies of the workload that steps rotate over, so that the "
+                         "bytes touched between two uses of one copy exceed the 256 MB Infinity Cache")
     return ap.parse_args()
 
 
@@ -91,23 +96,23 @@ class DeviceSet:
         self.ptrs = [self.dev.data_ptr() + o for o in offs]
 
 
-def stress_workload():
+def stress_workload(replicas):
+    """Returns counts, the host image of the tensors, and `replicas` (src, dst) device sets."""
     import torch
     from horovod_amd import workloads as W
     counts = W.stress_counts(seed=3)
     rng = np.random.default_rng(4)
     host = np.zeros(sum((c * 4 + 255) // 256 * 256 for c in counts), np.uint8)
-
-    def fill(nbytes):
-        off = 0
-        for c in counts:
-            host[off:off + 4 * c] = rng.uniform(-1, 1, c).astype(np.float32).view(np.uint8)
-            off += (c * 4 + 255) // 256 * 256
-        return torch.from_numpy(host).cuda()
-
-    src = DeviceSet(counts, 4, fill)
-    dst = DeviceSet(counts, 4, lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
-    return counts, host, src, dst
+    off = 0
+    for c in counts:
+        host[off:off + 4 * c] = rng.uniform(-1, 1, c).astype(np.float32).view(np.uint8)
+        off += (c * 4 + 255) // 256 * 256
+    sets = []
+    for _ in range(replicas):
+        src = DeviceSet(counts, 4, lambda n: torch.from_numpy(host).cuda())
+        dst = DeviceSet(counts, 4, lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
+        sets.append((src, dst))
+    return counts, host, sets
 
 
 def cpu_baseline_stress(counts, host, budget_s=12.0):
@@ -137,7 +142,7 @@ def cpu_baseline_stress(counts, host, budget_s=12.0):
         L.orc_unpack(c_void_p(buf.ctypes.data), optr, c_void_p(nb.ctypes.data), c_int(n))
         reps += 1
         dt = time.perf_counter() - t0
-        if dt > budget_s or reps >= 200:
+        if dt > budget_s:
             break
     gbs = 4 * payload * reps / dt / 1e9
     return {"value": round(gbs, 3), "unit": "GB/s", "cores": 1, "kind": "port",
@@ -159,63 +164,85 @@ def extras(steps, warmup):
         n = nbytes // torch.empty(0, dtype=dtype).element_size()
         return (torch.randn(n, generator=g, device="cuda", dtype=torch.float32) * std).to(dtype).view(torch.uint8)
 
-    def run_pipeline(name, shapes, tdtype, bdtype, std, peers, fraction, streams, kway=True, steps_=steps):
+    def run_pipeline(name, shapes, tdtype, bdtype, std, peers, fraction, streams, kway=True, steps_=steps,
+                     replicas=1):
         tt = {DTYPE["float32"]: torch.float32, DTYPE["float16"]: torch.float16}
         es = 4 if tdtype == DTYPE["float32"] else 2
         counts = [W.numel(s) for s in shapes]
-        src = DeviceSet(counts, es, lambda n: randn(n, tt[tdtype], std, 1))
-        dst = DeviceSet(counts, es, lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
-        pipe = AllreducePipeline(src.ptrs, dst.ptrs, counts, tdtype, bdtype, num_streams=streams)
-        bs = 4 if pipe.buffer_dtype == DTYPE["float32"] else 2
-        max_elems = max(c.buffer_elems for c in pipe.cycles)
-        peer_bufs = []
-        for p in range(peers):
-            nb = int(max_elems * fraction) * bs + 256
-            peer_bufs.append(randn((nb + 255) // 256 * 256, tt[pipe.buffer_dtype], std, 100 + p))
+        reps = []
+        for r in range(replicas):
+            src = DeviceSet(counts, es, lambda n: randn(n, tt[tdtype], std, 1 + r))
+            dst = DeviceSet(counts, es, lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
+            pipe = AllreducePipeline(src.ptrs, dst.ptrs, counts, tdtype, bdtype, num_streams=streams)
+            bs = 4 if pipe.buffer_dtype == DTYPE["float32"] else 2
+            max_elems = max(c.buffer_elems for c in pipe.cycles)
+            peer_bufs = []
+            for p in range(peers):
+                nb = int(max_elems * fraction) * bs + 256
+                peer_bufs.append(randn((nb + 255) // 256 * 256, tt[pipe.buffer_dtype], std, 100 + 16 * r + p))
+            reps.append((src, dst, pipe, peer_bufs))
         torch.cuda.synchronize()
-        fn = lambda: pipe.run(0.125, 1.0, (lambda ci, p: peer_bufs[p].data_ptr()) if peers else None,
-                              peers, fraction, kway)
-        sec = timed(fn, pipe.synchronize, steps_, max(2, warmup // 4))
+        turn = [0]
+
+        def fn():
+            i = turn[0] = (turn[0] + 1) % len(reps)
+            _, _, pipe, peer_bufs = reps[i]
+            pipe.run(0.125, 1.0, (lambda ci, p: peer_bufs[p].data_ptr()) if peers else None, peers, fraction, kway)
+
+        def sync():
+            for _, _, pipe, _ in reps:
+                pipe.synchronize()
+
+        sec = timed(fn, sync, steps_, max(2, warmup // 4))
+        pipe = reps[0][2]
         ab = pipe.algorithmic_bytes(peers, fraction, kway)
         out[name] = {"GB/s": round(ab / sec / 1e9, 1), "frac_of_hbm_peak": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4),
                      "ms": round(sec * 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1), "cycles": len(pipe.cycles),
-                     "streams": streams, "peers": peers, "reduce": "k-way" if kway else "per-peer"}
-        pipe.destroy()
-        del src, dst, peer_bufs
+                     "streams": streams, "peers": peers, "reduce": "k-way" if kway else "per-peer",
+                     "replicas_rotated": replicas}
+        for _, _, pipe, _ in reps:
+            pipe.destroy()
+        del reps
         torch.cuda.empty_cache()
 
     F32, F16 = DTYPE["float32"], DTYPE["float16"]
-    run_pipeline("resnet50_fp32_pack_scale_reduce_unpack", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0, 1)
+    run_pipeline("resnet50_fp32_pack_scale_reduce_unpack", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0, 1,
+                 replicas=4)
     run_pipeline("bert_large_fp32_to_fp16_7peers_eighth_chunk", W.bert_large_shapes(), F32, F16, 1e-4, 7, 0.125, 1,
                  steps_=max(5, steps // 10))
     run_pipeline("gpt2_xl_fp16_two_streams", W.gpt2_xl_shapes(), F16, F16, 1e-3, 1, 1.0, 2,
                  steps_=max(3, steps // 40))
 
-    # Adasum combine: two fp32 vectors of 2^25 elements, 64 layers, per-layer correlation 0.3
+    # Adasum combine: two fp32 vectors of 2^25 elements, 64 layers, per-layer correlation 0.3;
+    # four independent pairs are rotated so that no pair is still cached when its turn comes again
     n = 1 << 25
     counts = W.adasum_layer_counts(n, 64, seed=13)
-    g.manual_seed(14)
-    a = torch.randn(n, generator=g, device="cuda", dtype=torch.float32)
-    g.manual_seed(15)
-    b = 0.3 * a + (1 - 0.09) ** 0.5 * torch.randn(n, generator=g, device="cuda", dtype=torch.float32)
-    a0 = a.clone()
+    pairs = []
+    for r in range(4):
+        g.manual_seed(14 + 2 * r)
+        a = torch.randn(n, generator=g, device="cuda", dtype=torch.float32)
+        g.manual_seed(15 + 2 * r)
+        b = 0.3 * a + (1 - 0.09) ** 0.5 * torch.randn(n, generator=g, device="cuda", dtype=torch.float32)
+        pairs.append((a, b))
     plan = AdasumPlan(counts, F32)
     s = Stream()
     torch.cuda.synchronize()
+    turn = [0]
 
     def combine():
-        plan.combine(a.data_ptr(), b.data_ptr(), s)
+        # the combine rewrites a; its cost does not depend on the values, which stay finite
+        i = turn[0] = (turn[0] + 1) % len(pairs)
+        plan.combine(pairs[i][0].data_ptr(), pairs[i][1].data_ptr(), s)
 
-    # the combine rewrites a; its cost does not depend on the values, which stay finite:
-    # coefficients are <= 1 in magnitude for positively correlated pairs
-    sec = event_timed(combine, s, max(5, steps // 4), 3)
+    sec = event_timed(combine, s, max(8, steps // 4), 4)
     ab = 5 * n * 4
     out["adasum_fp32_2x32M_64layers"] = {"GB/s": round(ab / sec / 1e9, 1),
                                          "frac_of_hbm_peak": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4),
-                                         "ms": round(sec * 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1)}
+                                         "ms": round(sec * 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1),
+                                         "replicas_rotated": len(pairs)}
     plan.destroy()
     s.destroy()
-    del a, b, a0
+    del pairs
     return out
 
 
@@ -233,20 +260,35 @@ def main():
     from horovod_amd import DTYPE, FusionPlan, Stream
     horovod_amd.lib()  # fails loudly if the HIP library is not built
 
-    counts, host, src, dst = stress_workload()
-    F32 = DTYPE["float32"]
-    plan = FusionPlan(src.ptrs, dst.ptrs, counts, F32)
-    fb = torch.empty(plan.buffer_len, dtype=torch.uint8, device="cuda")
     stream = Stream()
+    F32 = DTYPE["float32"]
+    if args.calibrate:
+        from horovod_amd import host as H
+        n = 256 << 20
+        a = torch.zeros(n, dtype=torch.uint8, device="cuda")
+        b = torch.empty(n, dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        for _ in range(args.warmup + args.steps):
+            H.batched_d2d_memcpy([b.data_ptr()], [a.data_ptr()], [n], stream)
+        stream.synchronize()
+        return
+
+    counts, host, sets = stress_workload(max(1, args.replicas))
+    plans = [FusionPlan(src.ptrs, dst.ptrs, counts, F32) for src, dst in sets]
+    fbs = [torch.empty(plans[0].buffer_len, dtype=torch.uint8, device="cuda") for _ in sets]
+    plan = plans[0]
     payload = 4 * sum(counts)
     torch.cuda.synchronize()
+    turn = [0]
 
     def pack():
-        plan.pack(fb.data_ptr(), 0.125, stream)
+        i = turn[0] = (turn[0] + 1) % len(plans)
+        plans[i].pack(fbs[i].data_ptr(), 0.125, stream)
 
     def step():
-        plan.pack(fb.data_ptr(), 0.125, stream)
-        plan.unpack(fb.data_ptr(), 1.0, stream)
+        i = turn[0] = (turn[0] + 1) % len(plans)
+        plans[i].pack(fbs[i].data_ptr(), 0.125, stream)
+        plans[i].unpack(fbs[i].data_ptr(), 1.0, stream)
 
     if args.kernel_only:
         for _ in range(args.warmup + args.steps):
@@ -272,14 +314,15 @@ def main():
         "config": {"workload": "fusion stress: 1,024 fp32 tensors, log-uniform 256..65,536 elements (seed 3), "
                                "U(-1,1) (seed 4); pack with prescale 0.125 into a 64 MiB fusion buffer, unpack",
                    "tensors": len(counts), "payload_bytes": payload, "buffer_len": plan.buffer_len,
-                   "algorithmic_bytes_per_step": 4 * payload},
+                   "algorithmic_bytes_per_step": 4 * payload, "replicas_rotated": len(plans)},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "roofline": roofline,
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline_stress(counts, host)
-    plan.destroy()
-    del fb, src, dst
+    for p in plans:
+        p.destroy()
+    del fbs, sets
     torch.cuda.empty_cache()
     if not args.no_extra:
         result["extra"] = extras(args.steps, args.warmup)

@@ -28,7 +28,8 @@ class HvdHipError(RuntimeError):
 
 
 def lib_path():
-    return os.path.join(_HERE, "lib", "libhvdhip.so")
+    """The in-tree library, or the file named by HVDHIP_LIBRARY."""
+    return os.environ.get("HVDHIP_LIBRARY") or os.path.join(_HERE, "lib", "libhvdhip.so")
 
 
 _PV = POINTER(c_void_p)

@@ -30,9 +30,14 @@
 namespace hvdhip {
 namespace {
 
-// Layer table entry, stored in a Seg: off = first element of the layer,
-// n = its element count, output = index of its first chunk (= first partial
-// triple), tensor = number of chunks.
+// Chunk table entry as used here: tensor = index of the chunk's first element
+// in the vectors, output = layer number, n = elements in the chunk.
+//
+// Layer table entry: first partial triple of the layer and how many it has.
+struct Layer {
+  uint32_t first;
+  uint32_t count;
+};
 
 struct Triple {
   double d, a, b;
@@ -69,21 +74,16 @@ __device__ __forceinline__ Triple wg_reduce(Triple t) {
 constexpr int kUnroll = 4;
 
 template <typename T>
-__global__ __launch_bounds__(kWG) void dot_partials_k(const Seg* __restrict__ layers,
-                                                      const Chunk* __restrict__ chunks,
+__global__ __launch_bounds__(kWG) void dot_partials_k(const Chunk* __restrict__ chunks,
                                                       const T* __restrict__ a,
                                                       const T* __restrict__ b,
-                                                      uint32_t chunk_units,
                                                       double* __restrict__ partials) {
   constexpr int VEC = 16 / (int)sizeof(T);
   typedef Arr<T, VEC> V;
   const Chunk c = chunks[blockIdx.x];
-  const Seg L = layers[c.seg];
-  const uint64_t start = (uint64_t)c.idx * chunk_units;
-  const uint64_t left = L.n - start;
-  const uint32_t n = left < chunk_units ? (uint32_t)left : chunk_units;
-  gptr<const T> pa = as_global(a + L.off + start);
-  gptr<const T> pb = as_global(b + L.off + start);
+  const uint32_t n = c.n;
+  gptr<const T> pa = as_global(a + c.tensor);
+  gptr<const T> pb = as_global(b + c.tensor);
   const uint32_t nv = n / VEC;
   double d0 = 0., d1 = 0., a0 = 0., a1 = 0., b0 = 0., b1 = 0.;
   uint32_t v = threadIdx.x;
@@ -138,12 +138,12 @@ __global__ __launch_bounds__(kWG) void dot_partials_k(const Seg* __restrict__ la
 
 // One workgroup per layer: sums the layer's partial triples in a fixed order,
 // stores {dot, |a|^2, |b|^2} and the coefficients of adasum.h:397-404.
-__global__ __launch_bounds__(kWG) void finalize_k(const Seg* __restrict__ layers,
+__global__ __launch_bounds__(kWG) void finalize_k(const Layer* __restrict__ layers,
                                                   const double* __restrict__ partials,
                                                   double* __restrict__ normdots,
                                                   double* __restrict__ coeffs, double guard) {
-  const Seg L = layers[blockIdx.x];
-  const uint64_t first = L.output, count = L.tensor;
+  const Layer L = layers[blockIdx.x];
+  const uint64_t first = L.first, count = L.count;
   Triple t = {0., 0., 0.};
   for (uint64_t i = threadIdx.x; i < count; i += kWG) {
     t.d += partials[3 * (first + i) + 0];
@@ -181,24 +181,19 @@ struct Axpby<half_t> {
 };
 
 template <typename T>
-__global__ __launch_bounds__(kWG) void scaled_add_k(const Seg* __restrict__ layers,
-                                                    const Chunk* __restrict__ chunks, T* a,
+__global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ chunks, T* a,
                                                     const T* __restrict__ b,
-                                                    uint32_t chunk_units,
                                                     const double* __restrict__ coeffs,
                                                     double ca_arg, double cb_arg) {
   // coeffs == nullptr: every layer uses the by-value pair (ca_arg, cb_arg).
   constexpr int VEC = 16 / (int)sizeof(T);
   typedef Arr<T, VEC> V;
   const Chunk c = chunks[blockIdx.x];
-  const Seg L = layers[c.seg];
-  const double ca = coeffs ? coeffs[2 * (uint64_t)c.seg] : ca_arg;
-  const double cb = coeffs ? coeffs[2 * (uint64_t)c.seg + 1] : cb_arg;
-  const uint64_t start = (uint64_t)c.idx * chunk_units;
-  const uint64_t left = L.n - start;
-  const uint32_t n = left < chunk_units ? (uint32_t)left : chunk_units;
-  gptr<T> pa = as_global(a + L.off + start);
-  gptr<const T> pb = as_global(b + L.off + start);
+  const double ca = coeffs ? coeffs[2 * c.output] : ca_arg;
+  const double cb = coeffs ? coeffs[2 * c.output + 1] : cb_arg;
+  const uint32_t n = c.n;
+  gptr<T> pa = as_global(a + c.tensor);
+  gptr<const T> pb = as_global(b + c.tensor);
   const uint32_t nv = n / VEC;
   uint32_t v = threadIdx.x;
   for (; v + (kUnroll - 1) * kWG < nv; v += kUnroll * kWG) {
@@ -236,7 +231,8 @@ struct hvdhip_adasum_plan {
   int dtype = 0;
   int64_t total = 0;
   DevTables tables;
-  double* results = nullptr;  // one allocation: partials | normdots | coeffs
+  Layer* layers = nullptr;    // device, nlayers entries
+  double* results = nullptr;  // one allocation: partials | normdots | coeffs | layer table
   double* partials = nullptr;
   double* normdots = nullptr;
   double* coeffs = nullptr;
@@ -250,24 +246,21 @@ int plan_dot_norms(hvdhip_adasum_plan* p, const void* a, const void* b, hipStrea
   if (t.nchunks > 0) {
     switch (p->dtype) {
     case HVDHIP_FLOAT16:
-      hipLaunchKernelGGL((dot_partials_k<half_t>), dim3(t.nchunks), dim3(kWG), 0, s, t.segs, t.chunks,
-                         static_cast<const half_t*>(a), static_cast<const half_t*>(b), t.chunk_units,
-                         p->partials);
+      hipLaunchKernelGGL((dot_partials_k<half_t>), dim3(t.nchunks), dim3(kWG), 0, s, t.chunks,
+                         static_cast<const half_t*>(a), static_cast<const half_t*>(b), p->partials);
       break;
     case HVDHIP_FLOAT32:
-      hipLaunchKernelGGL((dot_partials_k<float>), dim3(t.nchunks), dim3(kWG), 0, s, t.segs, t.chunks,
-                         static_cast<const float*>(a), static_cast<const float*>(b), t.chunk_units,
-                         p->partials);
+      hipLaunchKernelGGL((dot_partials_k<float>), dim3(t.nchunks), dim3(kWG), 0, s, t.chunks,
+                         static_cast<const float*>(a), static_cast<const float*>(b), p->partials);
       break;
     default:
-      hipLaunchKernelGGL((dot_partials_k<double>), dim3(t.nchunks), dim3(kWG), 0, s, t.segs, t.chunks,
-                         static_cast<const double*>(a), static_cast<const double*>(b), t.chunk_units,
-                         p->partials);
+      hipLaunchKernelGGL((dot_partials_k<double>), dim3(t.nchunks), dim3(kWG), 0, s, t.chunks,
+                         static_cast<const double*>(a), static_cast<const double*>(b), p->partials);
       break;
     }
     HVDHIP_CHECK_LAUNCH("dot_partials_k");
   }
-  hipLaunchKernelGGL(finalize_k, dim3((uint32_t)p->nlayers), dim3(kWG), 0, s, t.segs, p->partials,
+  hipLaunchKernelGGL(finalize_k, dim3((uint32_t)p->nlayers), dim3(kWG), 0, s, p->layers, p->partials,
                      p->normdots, p->coeffs, std::sqrt(DBL_MIN));
   HVDHIP_CHECK_LAUNCH("finalize_k");
   return 0;
@@ -280,16 +273,16 @@ int plan_scaled_add(hvdhip_adasum_plan* p, void* a, const void* b, const double*
   if (t.nchunks == 0) return 0;
   switch (p->dtype) {
   case HVDHIP_FLOAT16:
-    hipLaunchKernelGGL((scaled_add_k<half_t>), dim3(t.nchunks), dim3(kWG), 0, s, t.segs, t.chunks,
-                       static_cast<half_t*>(a), static_cast<const half_t*>(b), t.chunk_units, coeffs, ca, cb);
+    hipLaunchKernelGGL((scaled_add_k<half_t>), dim3(t.nchunks), dim3(kWG), 0, s, t.chunks,
+                       static_cast<half_t*>(a), static_cast<const half_t*>(b), coeffs, ca, cb);
     break;
   case HVDHIP_FLOAT32:
-    hipLaunchKernelGGL((scaled_add_k<float>), dim3(t.nchunks), dim3(kWG), 0, s, t.segs, t.chunks,
-                       static_cast<float*>(a), static_cast<const float*>(b), t.chunk_units, coeffs, ca, cb);
+    hipLaunchKernelGGL((scaled_add_k<float>), dim3(t.nchunks), dim3(kWG), 0, s, t.chunks,
+                       static_cast<float*>(a), static_cast<const float*>(b), coeffs, ca, cb);
     break;
   default:
-    hipLaunchKernelGGL((scaled_add_k<double>), dim3(t.nchunks), dim3(kWG), 0, s, t.segs, t.chunks,
-                       static_cast<double*>(a), static_cast<const double*>(b), t.chunk_units, coeffs, ca, cb);
+    hipLaunchKernelGGL((scaled_add_k<double>), dim3(t.nchunks), dim3(kWG), 0, s, t.chunks,
+                       static_cast<double*>(a), static_cast<const double*>(b), coeffs, ca, cb);
     break;
   }
   HVDHIP_CHECK_LAUNCH("scaled_add_k");
@@ -350,36 +343,46 @@ int hvdhip_adasum_plan_create(const int* tensor_counts, int nlayers, int dtype,
   if (nlayers < 0 || (nlayers > 0 && !tensor_counts)) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "bad tensor_counts");
   if (dtype != HVDHIP_FLOAT16 && dtype != HVDHIP_FLOAT32 && dtype != HVDHIP_FLOAT64)
     return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE, "Adasum supports FLOAT16, FLOAT32 and FLOAT64, not dtype %d", dtype);
-  const uint32_t chunk_units = chunk_bytes() / (uint32_t)dtype_size(dtype);
-  std::vector<Seg> layers((size_t)nlayers);
-  uint64_t off = 0, first = 0;
+  const uint32_t chunk_units = chunk_bytes(Family::kAdasum) / (uint32_t)dtype_size(dtype);
+  std::vector<Layer> layers((size_t)nlayers);
+  std::vector<Chunk> chunks;
+  uint64_t off = 0;
   for (int i = 0; i < nlayers; ++i) {
     if (tensor_counts[i] < 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "tensor_counts[%d] is negative", i);
     const uint64_t n = (uint64_t)tensor_counts[i];
-    const uint64_t c = (n + chunk_units - 1) / chunk_units;
-    layers[(size_t)i] = Seg{c, first, off, n};
+    layers[(size_t)i].first = (uint32_t)chunks.size();
+    for (uint64_t start = 0; start < n; start += chunk_units) {
+      const uint64_t left = n - start;
+      chunks.push_back(Chunk{off + start, (uint64_t)i, 0, (uint32_t)(left < chunk_units ? left : chunk_units), 0});
+    }
+    layers[(size_t)i].count = (uint32_t)chunks.size() - layers[(size_t)i].first;
+    if (chunks.size() > 0x7fffffffull) return fail(HVDHIP_ERR_TOO_LARGE, "too many chunks");
     off += n;
-    first += c;
   }
   hvdhip_adasum_plan* p = new hvdhip_adasum_plan();
   p->nlayers = nlayers;
   p->dtype = dtype;
   p->total = (int64_t)off;
-  int rc = build_tables(layers, chunk_units, &p->tables);
+  int rc = upload_chunks(chunks, &p->tables);
   if (rc) {
     delete p;
     return rc;
   }
   const size_t ndoubles = 3 * (size_t)p->tables.nchunks + 5 * (size_t)nlayers + 8;
-  hipError_t e = hipMalloc(reinterpret_cast<void**>(&p->results), ndoubles * sizeof(double));
+  const size_t layer_bytes = (size_t)nlayers * sizeof(Layer);
+  hipError_t e = hipMalloc(reinterpret_cast<void**>(&p->results), ndoubles * sizeof(double) + layer_bytes);
   if (e == hipSuccess) e = hipMemset(p->results, 0, ndoubles * sizeof(double));
+  if (e == hipSuccess && nlayers > 0)
+    e = hipMemcpy(p->results + ndoubles, layers.data(), layer_bytes, hipMemcpyHostToDevice);
   if (e != hipSuccess) {
+    (void)hipGetLastError();
     if (p->results) (void)hipFree(p->results);
     free_tables(&p->tables);
     delete p;
     return fail(e == hipErrorOutOfMemory ? HVDHIP_ERR_OUT_OF_MEMORY : (int)e,
                 "allocating Adasum results failed: %s", hipGetErrorString(e));
   }
+  p->layers = reinterpret_cast<Layer*>(p->results + ndoubles);
   p->partials = p->results;
   p->normdots = p->partials + 3 * (size_t)p->tables.nchunks;
   p->coeffs = p->normdots + 3 * (size_t)nlayers;

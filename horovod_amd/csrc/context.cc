@@ -52,58 +52,72 @@ int ok() {
   return 0;
 }
 
-uint32_t chunk_bytes() {
-  static uint32_t v = [] {
+uint32_t chunk_bytes(Family f) {
+  static uint32_t forced = [] {
     const char* e = getenv("HVDHIP_CHUNK_BYTES");
     if (e) {
       long x = strtol(e, nullptr, 10);
       if (x >= 4096 && x <= (1 << 24) && x % 4096 == 0) return (uint32_t)x;
     }
-    return kDefaultChunkBytes;
+    return 0u;
   }();
-  return v;
+  if (forced) return forced;
+  switch (f) {
+  case Family::kXfer: return kXferChunkBytes;
+  case Family::kReduce: return kReduceChunkBytes;
+  default: return kAdasumChunkBytes;
+  }
 }
 
-int build_tables(const std::vector<Seg>& segs, uint32_t chunk_units, DevTables* out) {
-  if (chunk_units == 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "chunk_units is zero");
-  uint64_t nchunks = 0;
-  for (const Seg& s : segs) {
-    uint64_t c = (s.n + chunk_units - 1) / chunk_units;
-    if (c > 0xffffffffull) return fail(HVDHIP_ERR_TOO_LARGE, "a segment needs more than 2^32 chunks");
-    nchunks += c;
-  }
-  if (nchunks > 0x7fffffffull || segs.size() > 0x7fffffffull)
-    return fail(HVDHIP_ERR_TOO_LARGE, "plan needs %llu workgroups; the limit is 2^31-1",
-                (unsigned long long)nchunks);
-  size_t seg_bytes = (segs.size() * sizeof(Seg) + 255) & ~(size_t)255;
-  size_t chunk_bytes_total = nchunks * sizeof(Chunk);
-  size_t total = seg_bytes + chunk_bytes_total;
-  if (total == 0) total = 256;
-  std::vector<unsigned char> host(total, 0);
-  if (!segs.empty()) memcpy(host.data(), segs.data(), segs.size() * sizeof(Seg));
-  Chunk* hc = reinterpret_cast<Chunk*>(host.data() + seg_bytes);
-  uint64_t k = 0;
-  for (size_t i = 0; i < segs.size(); ++i) {
-    uint64_t c = (segs[i].n + chunk_units - 1) / chunk_units;
-    for (uint64_t j = 0; j < c; ++j) hc[k++] = Chunk{(uint32_t)i, (uint32_t)j};
-  }
+int upload_chunks(const std::vector<Chunk>& chunks, DevTables* out) {
+  if (chunks.size() > 0x7fffffffull)
+    return fail(HVDHIP_ERR_TOO_LARGE, "plan needs %zu workgroups; the limit is 2^31-1", chunks.size());
+  const size_t total = chunks.empty() ? 256 : chunks.size() * sizeof(Chunk);
   void* dev = nullptr;
   hipError_t e = hipMalloc(&dev, total);
-  if (e != hipSuccess)
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
     return fail(e == hipErrorOutOfMemory ? HVDHIP_ERR_OUT_OF_MEMORY : (int)e,
                 "hipMalloc of %zu table bytes failed: %s", total, hipGetErrorString(e));
-  e = hipMemcpy(dev, host.data(), total, hipMemcpyHostToDevice);
-  if (e != hipSuccess) {
-    (void)hipFree(dev);
-    return fail((int)e, "hipMemcpy of plan tables failed: %s", hipGetErrorString(e));
+  }
+  if (!chunks.empty()) {
+    e = hipMemcpy(dev, chunks.data(), total, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      (void)hipFree(dev);
+      return fail((int)e, "hipMemcpy of plan tables failed: %s", hipGetErrorString(e));
+    }
   }
   out->alloc = dev;
-  out->segs = reinterpret_cast<Seg*>(dev);
-  out->chunks = reinterpret_cast<Chunk*>(static_cast<unsigned char*>(dev) + seg_bytes);
-  out->nsegs = (uint32_t)segs.size();
-  out->nchunks = (uint32_t)nchunks;
-  out->chunk_units = chunk_units;
+  out->chunks = static_cast<Chunk*>(dev);
+  out->nchunks = (uint32_t)chunks.size();
   return 0;
+}
+
+int build_tables(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t tensor_es,
+                 uint32_t buffer_es, DevTables* out) {
+  if (chunk_units == 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "chunk_units is zero");
+  uint64_t nchunks = 0;
+  for (const Seg& s : segs) nchunks += (s.n + chunk_units - 1) / chunk_units;
+  if (nchunks > 0x7fffffffull)
+    return fail(HVDHIP_ERR_TOO_LARGE, "plan needs %llu workgroups; the limit is 2^31-1",
+                (unsigned long long)nchunks);
+  std::vector<Chunk> chunks;
+  chunks.reserve((size_t)nchunks);
+  for (const Seg& s : segs) {
+    for (uint64_t start = 0; start < s.n; start += chunk_units) {
+      const uint64_t left = s.n - start;
+      Chunk c;
+      c.tensor = s.tensor + start * tensor_es;
+      c.output = s.output + start * tensor_es;
+      c.off = s.off + start * buffer_es;
+      c.n = (uint32_t)(left < chunk_units ? left : chunk_units);
+      const uint64_t nbytes = s.n * buffer_es;
+      c.pad = left <= chunk_units ? (uint32_t)((16 - (nbytes & 15)) & 15) : 0;
+      chunks.push_back(c);
+    }
+  }
+  return upload_chunks(chunks, out);
 }
 
 int free_tables(DevTables* t) {

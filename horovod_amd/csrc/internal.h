@@ -52,14 +52,22 @@ inline int64_t dtype_size(int dtype) {
 // Threads per workgroup of every streaming kernel: four wave64 wavefronts.
 constexpr int kWG = 256;
 
-// Bytes of the wider side that one workgroup moves.  Read once from
-// HVDHIP_CHUNK_BYTES (a multiple of 4096), default kDefaultChunkBytes.
-constexpr uint32_t kDefaultChunkBytes = 32768;
-uint32_t chunk_bytes();
+// Bytes of the wider side that one workgroup moves.  Measured on MI355X with
+// buffers far larger than the 256 MB Infinity Cache: one 16-byte access per
+// lane and workgroup (4 KiB) with non-temporal hints streams at about 80 % of
+// the HBM peak, against about 70 % for 16-32 KiB per workgroup; the occupancy
+// of many small workgroups hides latency better than unrolling inside one.
+// The Adasum reduction pays a workgroup-wide tree per chunk and prefers 16 KiB.
+// HVDHIP_CHUNK_BYTES (a multiple of 4096) overrides all three, for tuning.
+enum class Family { kXfer, kReduce, kAdasum };
+constexpr uint32_t kXferChunkBytes = 4096;
+constexpr uint32_t kReduceChunkBytes = 4096;
+constexpr uint32_t kAdasumChunkBytes = 16384;
+uint32_t chunk_bytes(Family f);
 
-// One contiguous run of elements to transfer.  `tensor` and `output` are
-// absolute device addresses; `off` is a byte offset into the fusion buffer
-// whose base address is given at launch.  `n` counts elements.
+// One contiguous run of elements to transfer (host side only).  `tensor` and
+// `output` are absolute device addresses; `off` is a byte offset into the
+// fusion buffer whose base address is given at launch.  `n` counts elements.
 struct Seg {
   uint64_t tensor;
   uint64_t output;
@@ -67,27 +75,33 @@ struct Seg {
   uint64_t n;
 };
 
-// One workgroup's share: chunk number `idx` (in units of chunk_units
-// elements) of segment `seg`.
+// One workgroup's share, self-contained so that a workgroup needs a single
+// 32-byte scalar load before it can issue its data loads.  All three
+// locations already point at the chunk's first element.
 struct Chunk {
-  uint32_t seg;
-  uint32_t idx;
+  uint64_t tensor;  // absolute address on the tensor side
+  uint64_t output;  // absolute address on the output side
+  uint64_t off;     // byte offset into the fusion buffer
+  uint32_t n;       // elements in this chunk
+  uint32_t pad;     // bytes to zero after the chunk in the fusion buffer (last chunk of a tensor)
 };
+static_assert(sizeof(Chunk) == 32, "Chunk is loaded as eight dwords");
 
-// Device-resident segment and chunk tables of one plan.
+// Device-resident chunk table of one plan.
 struct DevTables {
-  void* alloc = nullptr;  // one allocation holding both tables
-  Seg* segs = nullptr;
+  void* alloc = nullptr;
   Chunk* chunks = nullptr;
-  uint32_t nsegs = 0;
   uint32_t nchunks = 0;
-  uint32_t chunk_units = 0;  // elements per chunk
 };
 
-// Builds the chunk table for `segs`, with chunk_units elements per chunk, and
-// uploads both tables (allocates; synchronous).  Zero-length segments get no
-// chunk.
-int build_tables(const std::vector<Seg>& segs, uint32_t chunk_units, DevTables* out);
+// Cuts every segment into chunks of at most chunk_units elements and uploads
+// the table (allocates; synchronous).  tensor_es / buffer_es are the element
+// sizes on the tensor/output side and on the fusion-buffer side.  Zero-length
+// segments get no chunk.
+int build_tables(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t tensor_es,
+                 uint32_t buffer_es, DevTables* out);
+// Uploads a ready-made chunk table.
+int upload_chunks(const std::vector<Chunk>& chunks, DevTables* out);
 int free_tables(DevTables* t);
 
 }  // namespace hvdhip

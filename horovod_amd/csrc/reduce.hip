@@ -93,7 +93,7 @@ __global__ __launch_bounds__(kWG) void reduce_k(T* resident, Peers<K> peers, uin
 template <typename T, int K>
 int launch_k(void* resident, const void* const* incoming, int64_t n, hipStream_t stream) {
   // Fewer bytes per workgroup as more peers stream in, to keep loads in flight similar.
-  uint32_t tile = chunk_bytes() / (uint32_t)sizeof(T);
+  uint32_t tile = chunk_bytes(Family::kReduce) / (uint32_t)sizeof(T);
   const uint64_t blocks = ((uint64_t)n + tile - 1) / tile;
   if (blocks > 0x7fffffffull) return fail(HVDHIP_ERR_TOO_LARGE, "chunk of %lld elements is too large", (long long)n);
   Peers<K> peers;

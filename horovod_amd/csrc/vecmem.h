@@ -60,17 +60,33 @@ struct Arr {
   T v[N];
 };
 
+// Streaming data is touched once: the non-temporal hint keeps it from
+// displacing useful lines in L2 and the Infinity Cache.
+#ifndef HVDHIP_NONTEMPORAL
+#define HVDHIP_NONTEMPORAL 1
+#endif
+
 template <typename T, int N>
 __device__ __forceinline__ Arr<T, N> ldv(gptr<const T> p) {
   typedef typename Raw<(int)sizeof(T) * N, (int)alignof(T)>::type R;
+#if HVDHIP_NONTEMPORAL
+  const typename RawSel<(int)sizeof(T) * N>::type r =
+      __builtin_nontemporal_load(reinterpret_cast<gptr<const R>>(p));
+#else
   const typename RawSel<(int)sizeof(T) * N>::type r = *reinterpret_cast<gptr<const R>>(p);
+#endif
   return __builtin_bit_cast(Arr<T, N>, r);
 }
 
 template <typename T, int N>
 __device__ __forceinline__ void stv(gptr<T> p, const Arr<T, N>& a) {
   typedef typename Raw<(int)sizeof(T) * N, (int)alignof(T)>::type R;
+#if HVDHIP_NONTEMPORAL
+  __builtin_nontemporal_store(__builtin_bit_cast(typename RawSel<(int)sizeof(T) * N>::type, a),
+                              reinterpret_cast<gptr<R>>(p));
+#else
   *reinterpret_cast<gptr<R>>(p) = __builtin_bit_cast(typename RawSel<(int)sizeof(T) * N>::type, a);
+#endif
 }
 
 }  // namespace hvdhip

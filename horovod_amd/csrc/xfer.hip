@@ -117,7 +117,10 @@ struct UnpackF16F32 {
   }
 };
 
-constexpr int kUnroll = 4;
+#ifndef HVDHIP_XFER_UNROLL
+#define HVDHIP_XFER_UNROLL 4
+#endif
+constexpr int kUnroll = HVDHIP_XFER_UNROLL;  // 16-byte loads in flight per lane
 
 // Streams n elements from src to dst through Op::f with the whole workgroup.
 template <class Op>
@@ -158,31 +161,20 @@ __device__ __forceinline__ void stream_range(gptr<const typename Op::S> src,
 enum Mode { kPack = 0, kUnpack = 1, kDirect = 2 };
 
 // One workgroup per chunk-table entry.
-//   kPack:   src = seg.tensor,        dst = base + seg.off (pad bytes zeroed)
-//   kUnpack: src = base + seg.off,    dst = seg.output
-//   kDirect: src = seg.tensor,        dst = seg.output
+//   kPack:   src = chunk.tensor,      dst = base + chunk.off (pad bytes zeroed)
+//   kUnpack: src = base + chunk.off,  dst = chunk.output
+//   kDirect: src = chunk.tensor,      dst = chunk.output
 template <class Op, int MODE>
-__global__ __launch_bounds__(kWG) void xfer_k(const Seg* __restrict__ segs,
-                                              const Chunk* __restrict__ chunks, uint64_t base,
-                                              uint32_t chunk_units, typename Op::P p) {
+__global__ __launch_bounds__(kWG) void xfer_k(const Chunk* __restrict__ chunks, uint64_t base,
+                                              typename Op::P p) {
   typedef typename Op::S S;
   typedef typename Op::D D;
   const Chunk c = chunks[blockIdx.x];
-  const Seg s = segs[c.seg];
-  const uint64_t start = (uint64_t)c.idx * chunk_units;
-  const uint64_t left = s.n - start;
-  const uint32_t n = left < chunk_units ? (uint32_t)left : chunk_units;
-  const uint64_t src_addr = (MODE == kUnpack) ? base + s.off : s.tensor;
-  const uint64_t dst_addr = (MODE == kPack) ? base + s.off : s.output;
-  gptr<const S> src = as_global<const S>(src_addr) + start;
-  gptr<D> dst = as_global<D>(dst_addr) + start;
-  stream_range<Op>(src, dst, n, p);
-  if (MODE == kPack && left <= chunk_units) {
-    // Last chunk of the tensor: zero the bytes up to the next 16-byte boundary.
-    const uint64_t nbytes = s.n * sizeof(D);
-    const uint32_t pad = (uint32_t)((16 - (nbytes & 15)) & 15);
-    if (threadIdx.x < pad) as_global<uint8_t>(dst_addr)[nbytes + threadIdx.x] = 0;
-  }
+  const uint64_t src_addr = (MODE == kUnpack) ? base + c.off : c.tensor;
+  const uint64_t dst_addr = (MODE == kPack) ? base + c.off : c.output;
+  stream_range<Op>(as_global<const S>(src_addr), as_global<D>(dst_addr), c.n, p);
+  if (MODE == kPack && threadIdx.x < c.pad)
+    as_global<uint8_t>(dst_addr)[(uint64_t)c.n * sizeof(D) + threadIdx.x] = 0;
 }
 
 // Contiguous buffer: workgroup b handles elements [b*tile, (b+1)*tile).
@@ -203,8 +195,7 @@ __global__ __launch_bounds__(kWG) void contig_k(const typename Op::S* src,
 template <class Op, int MODE>
 int launch_xfer(const DevTables& t, uint64_t base, typename Op::P p, hipStream_t stream) {
   if (t.nchunks == 0) return 0;
-  hipLaunchKernelGGL((xfer_k<Op, MODE>), dim3(t.nchunks), dim3(kWG), 0, stream, t.segs, t.chunks,
-                     base, t.chunk_units, p);
+  hipLaunchKernelGGL((xfer_k<Op, MODE>), dim3(t.nchunks), dim3(kWG), 0, stream, t.chunks, base, p);
   HVDHIP_CHECK_LAUNCH("xfer_k");
   return 0;
 }
@@ -246,7 +237,7 @@ bool scalable(int dtype) {
 
 template <class Op>
 int launch_contig(const void* in, void* out, int64_t n, typename Op::P p, hipStream_t stream) {
-  const uint32_t tile = chunk_bytes() / (uint32_t)std::max(sizeof(typename Op::S), sizeof(typename Op::D));
+  const uint32_t tile = chunk_bytes(Family::kXfer) / (uint32_t)std::max(sizeof(typename Op::S), sizeof(typename Op::D));
   const uint64_t blocks = ((uint64_t)n + tile - 1) / tile;
   if (blocks > 0x7fffffffull) return fail(HVDHIP_ERR_TOO_LARGE, "buffer of %lld elements is too large", (long long)n);
   hipLaunchKernelGGL((contig_k<Op>), dim3((uint32_t)blocks), dim3(kWG), 0, stream,
@@ -299,7 +290,7 @@ int cached_tables(void* const* out, const void* const* in, const size_t* sizes, 
     segs[i] = Seg{(uint64_t)(uintptr_t)in[i], (uint64_t)(uintptr_t)out[i], 0, sizes[i] / unit};
   CachedCopy entry;
   entry.key.swap(key);
-  int rc = build_tables(segs, chunk_bytes() / unit, &entry.tables);
+  int rc = build_tables(segs, chunk_bytes(Family::kXfer) / unit, unit, unit, &entry.tables);
   if (rc) return rc;
   if (c.lru.size() >= kCopyCacheCapacity) {
     // Tables may still be read by queued kernels: wait before freeing.
@@ -433,7 +424,7 @@ int hvdhip_fusion_plan_create(const void* const* tensors, void* const* outputs,
   p->buffer_dtype = buffer_dtype;
   p->buffer_len = off;
   p->offsets.swap(offsets);
-  int rc = build_tables(segs, chunk_bytes() / (uint32_t)std::max(ts, bs), &p->tables);
+  int rc = build_tables(segs, chunk_bytes(Family::kXfer) / (uint32_t)std::max(ts, bs), (uint32_t)ts, (uint32_t)bs, &p->tables);
   if (rc) {
     delete p;
     return rc;
