@@ -29,6 +29,12 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch of the scaled pack kernel on the headline workload, from rocprofv3
+# FETCH_SIZE and WRITE_SIZE runs of `bench.py --kernel-only`, each scaled by what the same
+# counter reads for a plain 256 MiB copy (`bench.py --calibrate`): FETCH_SIZE x 1.9544,
+# WRITE_SIZE x 1.0000.  The summary with the commands is profiles/pack_kernel_fusion_stress.txt.
+PACK_TRAFFIC_BYTES_MEASURED = 93107696
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -302,7 +308,7 @@ def main():
     ksec = event_timed(pack, stream, args.steps, args.warmup)
     achieved = 2 * payload / ksec / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": PACK_TRAFFIC_BYTES_MEASURED,
                 "kernel": "xfer_k<Scale<float,float>, pack>", "launch_us": round(ksec * 1e6, 2),
                 "algorithmic_bytes_per_launch": 2 * payload, "workgroups": plan.num_chunks}
 
