@@ -1,0 +1,126 @@
+// adapter_capi.cc -- a small C surface over the adapter classes so that the
+// Python tests can drive them (exceptions are turned into a message buffer).
+#include <cstring>
+#include <stdexcept>
+
+#include "hvd_hip_adapter.h"
+
+using namespace horovod::common;
+
+namespace {
+struct Harness {
+  GPUContext context;
+  GlobalState state;
+  GPUAllreduce* allreduce = nullptr;
+  AdasumGPU* adasum = nullptr;
+};
+
+int report(const std::exception& e, char* err, size_t errlen) {
+  if (err && errlen) {
+    std::strncpy(err, e.what(), errlen - 1);
+    err[errlen - 1] = 0;
+  }
+  return -1;
+}
+}  // namespace
+
+extern "C" {
+
+void* hvd_adapter_create(int num_streams, int batch_d2d_memcopies, int enable_async_completion, int elastic,
+                         void* const* fusion_buffers) {
+  Harness* h = new Harness();
+  h->state.num_nccl_streams = num_streams;
+  h->state.batch_d2d_memcopies = batch_d2d_memcopies != 0;
+  h->state.enable_async_completion = enable_async_completion != 0;
+  h->state.elastic_enabled = elastic != 0;
+  for (int i = 0; i < num_streams; ++i) h->state.fusion_buffer.push_back(fusion_buffers[i]);
+  h->allreduce = new GPUAllreduce(&h->context, &h->state);
+  h->adasum = new AdasumGPU(&h->context);
+  return h;
+}
+
+void hvd_adapter_destroy(void* handle) {
+  Harness* h = static_cast<Harness*>(handle);
+  if (!h) return;
+  delete h->allreduce;
+  delete h->adasum;
+  for (auto& m : h->context.streams)
+    for (auto& kv : m)
+      if (kv.second) hvdhip_stream_destroy(kv.second);
+  delete h;
+}
+
+int hvd_adapter_allreduce(void* handle, const void* const* tensors, void* const* outputs, const int64_t* counts,
+                          int n, int dtype, double prescale, double postscale, const void* const* peers,
+                          int npeers, char* err, size_t errlen) {
+  Harness* h = static_cast<Harness*>(handle);
+  try {
+    std::vector<TensorTableEntry> entries((size_t)n);
+    for (int i = 0; i < n; ++i) {
+      entries[(size_t)i].tensor_name = "t" + std::to_string(i);
+      entries[(size_t)i].tensor_data = tensors[i];
+      entries[(size_t)i].output_data = outputs[i];
+      entries[(size_t)i].num_elements = counts[i];
+      entries[(size_t)i].dtype = (DataType)dtype;
+      entries[(size_t)i].device = 0;
+    }
+    std::vector<const void*> p(peers, peers + npeers);
+    h->allreduce->Execute(entries, prescale, postscale, p);
+    return 0;
+  } catch (const std::exception& e) {
+    return report(e, err, errlen);
+  }
+}
+
+int hvd_adapter_state(void* handle, int* current_stream, int* cached_plans) {
+  Harness* h = static_cast<Harness*>(handle);
+  *current_stream = h->state.current_nccl_stream;
+  *cached_plans = (int)h->allreduce->cached_plans();
+  return 0;
+}
+
+int hvd_adapter_adasum_pairwise(void* handle, void* a, const void* b, int dtype, const int* counts, int nlayers,
+                                double* normdots, char* err, size_t errlen) {
+  Harness* h = static_cast<Harness*>(handle);
+  try {
+    gpuStream_t s = nullptr;
+    if (h->context.streams.empty()) h->context.streams.resize(1);
+    gpuStream_t& slot = h->context.streams[0][0];
+    if (!slot) h->context.StreamCreate(&slot);
+    s = slot;
+    std::vector<int> tc(counts, counts + nlayers);
+    std::vector<double> nd;
+    h->adasum->FusedPairwiseReduce(a, b, (DataType)dtype, tc, &nd, s);
+    if (normdots) std::memcpy(normdots, nd.data(), nd.size() * sizeof(double));
+    h->context.StreamSynchronize(s);
+    return 0;
+  } catch (const std::exception& e) {
+    return report(e, err, errlen);
+  }
+}
+
+int hvd_adapter_adasum_dispatch(void* handle, void* a, void* b, int dtype, int count, double* out3, double acoeff,
+                                double bcoeff, char* err, size_t errlen) {
+  Harness* h = static_cast<Harness*>(handle);
+  try {
+    if (h->context.streams.empty()) h->context.streams.resize(1);
+    gpuStream_t& s = h->context.streams[0][0];
+    if (!s) h->context.StreamCreate(&s);
+    h->adasum->DispatchComputeDotAndNormSqrds(a, b, (DataType)dtype, count, out3[0], out3[1], out3[2], s);
+    h->adasum->DispatchScaledAdd((DataType)dtype, count, acoeff, a, bcoeff, b, s);
+    h->context.StreamSynchronize(s);
+    return 0;
+  } catch (const std::exception& e) {
+    return report(e, err, errlen);
+  }
+}
+
+int hvd_adapter_fuse(const int64_t* tensor_bytes, int n, int64_t threshold, int batch_d2d_memcopies, int* group_of) {
+  std::vector<int64_t> tb(tensor_bytes, tensor_bytes + n);
+  auto groups = FuseResponses(tb, threshold, batch_d2d_memcopies != 0);
+  for (size_t g = 0; g < groups.size(); ++g)
+    for (int i : groups[g]) group_of[i] = (int)g;
+  return (int)groups.size();
+}
+
+}  // extern "C"

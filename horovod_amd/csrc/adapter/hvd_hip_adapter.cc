@@ -1,0 +1,395 @@
+// hvd_hip_adapter.cc -- see hvd_hip_adapter.h.  Host code; links only libhvdhip.so.
+#include "hvd_hip_adapter.h"
+
+#include <stdexcept>
+#include <thread>
+
+namespace horovod {
+namespace common {
+
+std::size_t DataType_Size(DataType value) {
+  int64_t s = hvdhip_dtype_size((int)value);
+  if (s < 0) throw std::logic_error("Type " + DataType_Name(value) + " is not supported.");
+  return (std::size_t)s;
+}
+
+const std::string& DataType_Name(DataType value) {
+  static const std::string names[] = {"uint8", "int8", "uint16", "int16", "int32", "int64",
+                                      "float16", "float32", "float64", "bool"};
+  static const std::string unknown("<unknown>");
+  return ((int)value >= 0 && (int)value <= 9) ? names[(int)value] : unknown;
+}
+
+// ---------------------------------------------------------------- GPUContext
+
+GPUContext::GPUContext() {}
+GPUContext::~GPUContext() {}
+
+void GPUContext::ErrorCheck(std::string op_name, int gpu_result) {
+  if (gpu_result != 0) {
+    std::string detail = hvdhip_last_error();
+    throw std::logic_error(op_name + " failed: " + hvdhip_error_string(gpu_result) +
+                           (detail.empty() ? "" : " (" + detail + ")"));
+  }
+}
+
+static Event AcquireEvent(GPUContext* ctx, gpuStream_t stream) {
+  void* ev = nullptr;
+  ctx->ErrorCheck("GetGpuEvent", hvdhip_event_acquire(stream, &ev));
+  Event event;
+  event.event = std::make_shared<void*>(ev);
+  event.stream = stream;
+  return event;
+}
+
+void GPUContext::RecordEvent(std::queue<std::pair<std::string, Event>>& event_queue, std::string name,
+                             gpuStream_t& stream) {
+  Event event = AcquireEvent(this, stream);
+  ErrorCheck("hipEventRecord", hvdhip_event_record(*event.event, event.stream));
+  event_queue.emplace(name, event);
+}
+
+Event GPUContext::RecordEvent(gpuStream_t& stream) {
+  Event event = AcquireEvent(this, stream);
+  ErrorCheck("hipEventRecord", hvdhip_event_record(*event.event, event.stream));
+  return event;
+}
+
+void GPUContext::ReleaseEvent(Event event) {
+  ErrorCheck("ReleaseGpuEvent", hvdhip_event_release(event.stream, *event.event));
+}
+
+void GPUContext::WaitForEvents(std::queue<std::pair<std::string, Event>>& event_queue,
+                               const std::function<void()>& error_check_callback, bool elastic) {
+  while (!event_queue.empty()) {
+    Event event = event_queue.front().second;
+    event_queue.pop();
+    if (elastic) {
+      // ops/cuda_operations.cc:116-132: poll, checking for asynchronous errors in between
+      while (true) {
+        int done = 0;
+        int rc = hvdhip_event_query(*event.event, &done);
+        if (rc != 0) throw std::logic_error(std::string("hipEventQuery failed: ") + hvdhip_error_string(rc));
+        if (done) break;
+        if (error_check_callback) error_check_callback();
+        std::this_thread::yield();
+      }
+    } else {
+      int rc = hvdhip_event_synchronize(*event.event);
+      if (rc != 0) throw std::logic_error(std::string("hipEventSynchronize failed: ") + hvdhip_error_string(rc));
+      if (error_check_callback) error_check_callback();
+    }
+    ErrorCheck("ReleaseGpuEvent", hvdhip_event_release(event.stream, *event.event));
+  }
+}
+
+void GPUContext::ClearEvents(std::queue<std::pair<std::string, Event>>& event_queue) {
+  while (!event_queue.empty()) {
+    Event event = event_queue.front().second;
+    event_queue.pop();
+    ErrorCheck("ReleaseGpuEvent", hvdhip_event_release(event.stream, *event.event));
+  }
+}
+
+void GPUContext::StreamCreate(gpuStream_t* stream) { ErrorCheck("hipStreamCreate", hvdhip_stream_create(stream)); }
+void GPUContext::StreamSynchronize(gpuStream_t stream) {
+  ErrorCheck("hipStreamSynchronize", hvdhip_stream_synchronize(stream));
+}
+int GPUContext::GetDevice() {
+  int device = 0;
+  ErrorCheck("hipGetDevice", hvdhip_get_device(&device));
+  return device;
+}
+void GPUContext::SetDevice(int device) { ErrorCheck("hipSetDevice", hvdhip_set_device(device)); }
+void GPUContext::MemcpyAsyncD2D(void* dst, const void* src, size_t count, gpuStream_t stream) {
+  ErrorCheck("hipMemcpyAsync", hvdhip_memcpy_async(dst, src, count, HVDHIP_MEMCPY_D2D, stream));
+}
+void GPUContext::MemcpyAsyncH2D(void* dst, const void* src, size_t count, gpuStream_t stream) {
+  ErrorCheck("hipMemcpyAsync", hvdhip_memcpy_async(dst, src, count, HVDHIP_MEMCPY_H2D, stream));
+}
+void GPUContext::MemcpyAsyncD2H(void* dst, const void* src, size_t count, gpuStream_t stream) {
+  ErrorCheck("hipMemcpyAsync", hvdhip_memcpy_async(dst, src, count, HVDHIP_MEMCPY_D2H, stream));
+}
+void GPUContext::ScaleBufferImpl(const void* fused_input_data, void* buffer_data, int64_t num_elements,
+                                 double scale_factor, DataType dtype, gpuStream_t stream) {
+  int rc = hvdhip_scale_buffer(fused_input_data, buffer_data, num_elements, scale_factor, (int)dtype, stream);
+  if (rc == HVDHIP_ERR_UNSUPPORTED_DTYPE)  // ops/cuda/cuda_kernels.cu:182-185
+    throw std::logic_error("Type " + DataType_Name(dtype) + " not supported by ScaleBufferCudaImpl.");
+  ErrorCheck("ScaleBufferImpl", rc);
+}
+
+// -------------------------------------------------------------- GPUOpContext
+
+GPUOpContext::GPUOpContext(GPUContext* context, GlobalState* global_state)
+    : gpu_context_(context), global_state_(global_state) {}
+
+void GPUOpContext::InitGPU(const std::vector<TensorTableEntry>& entries) {
+  auto& first_entry = entries[0];
+  gpu_context_->SetDevice(first_entry.device);
+  if (gpu_context_->streams.size() < (size_t)global_state_->num_nccl_streams)
+    gpu_context_->streams.resize((size_t)global_state_->num_nccl_streams);
+  gpuStream_t& s = gpu_context_->streams[(size_t)global_state_->current_nccl_stream][first_entry.device];
+  if (s == nullptr) gpu_context_->StreamCreate(&s);
+}
+
+void GPUOpContext::InitGPUQueue(const std::vector<TensorTableEntry>& entries) {
+  event_queue = std::queue<std::pair<std::string, Event>>();
+  stream = &gpu_context_->streams[(size_t)global_state_->current_nccl_stream][entries[0].device];
+}
+
+void GPUOpContext::FinalizeGPUQueue(std::vector<TensorTableEntry>& entries,
+                                    const std::function<void()>& error_check_callback) {
+  if (!global_state_->enable_async_completion) gpu_context_->RecordEvent(event_queue, "", *stream);
+  gpu_context_->SetDevice(entries[0].device);
+  if (!global_state_->enable_async_completion) {
+    gpu_context_->WaitForEvents(event_queue, error_check_callback, global_state_->elastic_enabled);
+  } else {
+    gpu_context_->ClearEvents(event_queue);
+    Event event = gpu_context_->RecordEvent(*stream);  // handed to the framework in Status.event
+    gpu_context_->ReleaseEvent(event);
+  }
+  global_state_->current_nccl_stream = (global_state_->current_nccl_stream + 1) % global_state_->num_nccl_streams;
+}
+
+// -------------------------------------------------------------- GPUAllreduce
+
+GPUAllreduce::GPUAllreduce(GPUContext* context, GlobalState* global_state)
+    : gpu_context_(context), global_state_(global_state), gpu_op_context_(context, global_state) {}
+
+GPUAllreduce::~GPUAllreduce() {
+  for (auto& kv : plans_) hvdhip_fusion_plan_destroy(kv.second);
+}
+
+gpuStream_t GPUAllreduce::Stream(const std::vector<TensorTableEntry>& entries) {
+  return gpu_context_->streams[(size_t)global_state_->current_nccl_stream][entries[0].device];
+}
+
+hvdhip_fusion_plan* GPUAllreduce::PlanFor(const std::vector<TensorTableEntry>& entries) {
+  std::vector<uint64_t> key;
+  key.reserve(3 * entries.size() + 1);
+  key.push_back((uint64_t)entries[0].dtype);
+  for (auto& e : entries) {
+    key.push_back((uint64_t)(uintptr_t)e.tensor_data);
+    key.push_back((uint64_t)(uintptr_t)e.output_data);
+    key.push_back((uint64_t)e.num_elements);
+  }
+  auto it = plans_.find(key);
+  if (it != plans_.end()) return it->second;
+  std::vector<const void*> tensors;
+  std::vector<void*> outputs;
+  std::vector<int64_t> counts;
+  for (auto& e : entries) {
+    tensors.push_back(e.tensor_data);
+    outputs.push_back(e.output_data);
+    counts.push_back(e.num_elements);
+  }
+  hvdhip_fusion_plan* plan = nullptr;
+  gpu_context_->ErrorCheck("hvdhip_fusion_plan_create",
+                           hvdhip_fusion_plan_create(tensors.data(), outputs.data(), counts.data(), (int)entries.size(),
+                                                     (int)entries[0].dtype, (int)entries[0].dtype, &plan));
+  plans_[key] = plan;
+  return plan;
+}
+
+void GPUAllreduce::MemcpyInFusionBuffer(const std::vector<TensorTableEntry>& entries,
+                                        const void*& fused_input_data, void*& buffer_data, size_t& buffer_len) {
+  ScaleMemcpyInFusionBuffer(entries, fused_input_data, buffer_data, buffer_len, 1.0);
+}
+
+void GPUAllreduce::ScaleMemcpyInFusionBuffer(const std::vector<TensorTableEntry>& entries,
+                                             const void*& fused_input_data, void*& buffer_data,
+                                             size_t& buffer_len, double scale_factor) {
+  buffer_data = global_state_->fusion_buffer[(size_t)global_state_->current_nccl_stream];
+  if (global_state_->batch_d2d_memcopies) {
+    hvdhip_fusion_plan* plan = PlanFor(entries);
+    int rc = hvdhip_fusion_pack(plan, buffer_data, scale_factor, HVDHIP_PACK_DEFAULT, Stream(entries));
+    if (rc == HVDHIP_ERR_UNSUPPORTED_DTYPE)  // ops/cuda/cuda_kernels.cu:317-319
+      throw std::logic_error("Type " + DataType_Name(entries[0].dtype) +
+                             " not supported by BatchedScaledD2DMemcpyCudaImpl.");
+    gpu_context_->ErrorCheck("BatchedScaledD2DMemcpyCudaImpl", rc);
+    buffer_len = (size_t)hvdhip_fusion_plan_buffer_len(plan);
+  } else {
+    // ops/gpu_operations.cc:209-222: one async copy per entry at unpadded offsets, then a whole-buffer scale
+    int64_t offset = 0;
+    for (auto& e : entries) {
+      MemcpyEntryInFusionBuffer(entries, e, (uint8_t*)buffer_data + offset);
+      offset += e.tensor_size();
+    }
+    buffer_len = (size_t)offset;
+    if (scale_factor != 1.0)
+      ScaleBuffer(scale_factor, entries, buffer_data, buffer_data,
+                  (int64_t)(buffer_len / DataType_Size(entries[0].dtype)));
+  }
+  fused_input_data = buffer_data;
+}
+
+void GPUAllreduce::MemcpyOutFusionBuffer(const void* buffer_data, std::vector<TensorTableEntry>& entries) {
+  ScaleMemcpyOutFusionBuffer(const_cast<void*>(buffer_data), 0, 1.0, entries);
+}
+
+void GPUAllreduce::ScaleMemcpyOutFusionBuffer(void* buffer_data, size_t buffer_len, double scale_factor,
+                                              std::vector<TensorTableEntry>& entries) {
+  if (global_state_->batch_d2d_memcopies) {
+    hvdhip_fusion_plan* plan = PlanFor(entries);
+    int rc = hvdhip_fusion_unpack(plan, buffer_data, scale_factor, Stream(entries));
+    if (rc == HVDHIP_ERR_UNSUPPORTED_DTYPE)
+      throw std::logic_error("Type " + DataType_Name(entries[0].dtype) +
+                             " not supported by BatchedScaledD2DMemcpyCudaImpl.");
+    gpu_context_->ErrorCheck("BatchedScaledD2DMemcpyCudaImpl", rc);
+  } else {
+    if (scale_factor != 1.0)
+      ScaleBuffer(scale_factor, entries, buffer_data, buffer_data,
+                  (int64_t)(buffer_len / DataType_Size(entries[0].dtype)));
+    int64_t offset = 0;
+    for (auto& e : entries) {
+      MemcpyEntryOutFusionBuffer(entries, (uint8_t*)buffer_data + offset, e);
+      offset += e.tensor_size();
+    }
+  }
+}
+
+void GPUAllreduce::MemcpyEntryInFusionBuffer(const std::vector<TensorTableEntry>& entries,
+                                             const TensorTableEntry& e, void* buffer_data_at_offset) {
+  gpu_context_->MemcpyAsyncD2D(buffer_data_at_offset, e.tensor_data, (size_t)e.tensor_size(), Stream(entries));
+}
+
+void GPUAllreduce::MemcpyEntryOutFusionBuffer(const std::vector<TensorTableEntry>& entries,
+                                              const void* buffer_data_at_offset, TensorTableEntry& e) {
+  gpu_context_->MemcpyAsyncD2D(e.output_data, buffer_data_at_offset, (size_t)e.tensor_size(), Stream(entries));
+}
+
+void GPUAllreduce::ScaleBuffer(double scale_factor, const std::vector<TensorTableEntry>& entries,
+                               const void* fused_input_data, void* buffer_data, int64_t num_elements) {
+  gpu_context_->ScaleBufferImpl(fused_input_data, buffer_data, num_elements, scale_factor, entries[0].dtype,
+                                Stream(entries));
+}
+
+void GPUAllreduce::Execute(std::vector<TensorTableEntry>& entries, double prescale_factor,
+                           double postscale_factor, const std::vector<const void*>& peers) {
+  auto& first_entry = entries[0];
+  gpu_op_context_.InitGPU(entries);
+  gpu_op_context_.InitGPUQueue(entries);
+  const void* fused_input_data;
+  void* buffer_data;
+  size_t buffer_len;
+  if (entries.size() > 1) {
+    ScaleMemcpyInFusionBuffer(entries, fused_input_data, buffer_data, buffer_len, prescale_factor);
+  } else {
+    // ops/nccl_operations.cc:176-186: no fusion buffer, tensor -> output
+    fused_input_data = first_entry.tensor_data;
+    buffer_data = first_entry.output_data;
+    buffer_len = (size_t)first_entry.tensor_size();
+    int64_t num_elements = first_entry.num_elements;
+    if (prescale_factor != 1.0) {
+      ScaleBuffer(prescale_factor, entries, fused_input_data, buffer_data, num_elements);
+      fused_input_data = buffer_data;
+    } else if (fused_input_data != buffer_data) {
+      gpu_context_->MemcpyAsyncD2D(buffer_data, fused_input_data, buffer_len, Stream(entries));
+    }
+  }
+  // The collective (ncclAllReduce(sum), ops/nccl_operations.cc:190-193) on one GPU.
+  if (!peers.empty()) {
+    int64_t num_elements = (int64_t)(buffer_len / DataType_Size(first_entry.dtype));
+    size_t done = 0;
+    while (done < peers.size()) {
+      int k = (int)std::min<size_t>(16, peers.size() - done);
+      gpu_context_->ErrorCheck("hvdhip_reduce_sum_k",
+                               hvdhip_reduce_sum_k(buffer_data, peers.data() + done, k, num_elements,
+                                                   (int)first_entry.dtype, Stream(entries)));
+      done += (size_t)k;
+    }
+  }
+  if (entries.size() > 1) {
+    ScaleMemcpyOutFusionBuffer(buffer_data, buffer_len, postscale_factor, entries);
+  } else if (postscale_factor != 1.0) {
+    ScaleBuffer(postscale_factor, entries, buffer_data, buffer_data, first_entry.num_elements);
+  }
+  gpu_op_context_.FinalizeGPUQueue(entries);
+}
+
+// ------------------------------------------------------------------ AdasumGPU
+
+AdasumGPU::AdasumGPU(GPUContext* context) : gpu_context_(context) {}
+AdasumGPU::~AdasumGPU() {
+  for (auto& kv : plans_) hvdhip_adasum_plan_destroy(kv.second);
+}
+
+static void CheckAdasumType(DataType t, const char* what) {
+  // ops/adasum/adasum.h:118-121,136-139
+  if (t != HOROVOD_FLOAT16 && t != HOROVOD_FLOAT32 && t != HOROVOD_FLOAT64)
+    throw std::logic_error(std::string("Unsupported data type in ") + what + ".");
+}
+
+void AdasumGPU::DispatchComputeDotAndNormSqrds(const void* a, const void* b, DataType horovod_datatype,
+                                               int count, double& dotProduct, double& anormsq,
+                                               double& bnormsq, gpuStream_t stream) {
+  CheckAdasumType(horovod_datatype, "ComputeDotAndNormSqrds");
+  gpu_context_->ErrorCheck("hvdhip_adasum_dot_and_norm_sqrds",
+                           hvdhip_adasum_dot_and_norm_sqrds(a, b, (int)horovod_datatype, count, &dotProduct,
+                                                            &anormsq, &bnormsq, stream));
+}
+
+void AdasumGPU::DispatchScaledAdd(DataType horovod_datatype, int count, double acoeff, void* a,
+                                  double bcoeff, void* b, gpuStream_t stream) {
+  CheckAdasumType(horovod_datatype, "ScaledAdd");
+  gpu_context_->ErrorCheck("hvdhip_adasum_dispatch_scaled_add",
+                           hvdhip_adasum_dispatch_scaled_add((int)horovod_datatype, count, acoeff, a, bcoeff, b,
+                                                             stream));
+}
+
+void AdasumGPU::FusedPairwiseReduce(void* a, const void* b, DataType horovod_datatype,
+                                    const std::vector<int>& tensor_counts, std::vector<double>* normAndDots,
+                                    gpuStream_t stream) {
+  CheckAdasumType(horovod_datatype, "FusedPairwiseReduce");
+  auto key = std::make_pair((int)horovod_datatype, tensor_counts);
+  hvdhip_adasum_plan* plan;
+  auto it = plans_.find(key);
+  if (it == plans_.end()) {
+    plan = nullptr;
+    gpu_context_->ErrorCheck("hvdhip_adasum_plan_create",
+                             hvdhip_adasum_plan_create(tensor_counts.data(), (int)tensor_counts.size(),
+                                                       (int)horovod_datatype, &plan));
+    plans_[key] = plan;
+  } else {
+    plan = it->second;
+  }
+  gpu_context_->ErrorCheck("hvdhip_adasum_combine", hvdhip_adasum_combine(plan, a, b, stream));
+  if (normAndDots) {
+    normAndDots->resize(3 * tensor_counts.size());
+    gpu_context_->ErrorCheck("hvdhip_adasum_read", hvdhip_adasum_read(plan, normAndDots->data(), nullptr, stream));
+  }
+}
+
+// -------------------------------------------------------------- FuseResponses
+
+std::vector<std::vector<int>> FuseResponses(const std::vector<int64_t>& tensor_bytes,
+                                            int64_t fusion_threshold_bytes, bool batch_d2d_memcopies) {
+  auto padded = [&](int64_t s) { return batch_d2d_memcopies ? 16 * ((s + 15) / 16) : s; };
+  const int n = (int)tensor_bytes.size();
+  std::vector<int> group_of((size_t)n, -1);
+  std::vector<std::vector<int>> groups;
+  for (int head = 0; head < n; ++head) {
+    if (group_of[(size_t)head] != -1) continue;
+    const int g = (int)groups.size();
+    groups.push_back({head});
+    group_of[(size_t)head] = g;
+    int64_t tensor_size = padded(tensor_bytes[(size_t)head]);
+    int64_t skipped_size = 0;
+    for (int j = head + 1; j < n; ++j) {
+      if (group_of[(size_t)j] != -1) continue;
+      const int64_t new_tensor_size = padded(tensor_bytes[(size_t)j]);
+      if (tensor_size + new_tensor_size <= fusion_threshold_bytes) {
+        tensor_size += new_tensor_size;
+        group_of[(size_t)j] = g;
+        groups[(size_t)g].push_back(j);
+      } else {
+        skipped_size += new_tensor_size;
+        if (tensor_size + skipped_size > fusion_threshold_bytes) break;
+      }
+    }
+  }
+  return groups;
+}
+
+}  // namespace common
+}  // namespace horovod

@@ -1,0 +1,192 @@
+// hvd_hip_adapter.h -- the host side above the C ABI: C++ classes shaped like
+// the reference's op layer for this path, calling nothing but include/hvdhip.h.
+//
+// These are the bodies a Horovod maintainer would put behind the existing
+// declarations (names, argument meaning and error behaviour are the
+// reference's):
+//   GPUContext          ops/gpu_operations.h:44-106, impl ops/cuda_operations.cc:28-210
+//   GPUOpContext        ops/gpu_operations.h:108-137, ops/gpu_operations.cc:27-106
+//   GPUAllreduce hooks  ops/gpu_operations.h:139-172, ops/gpu_operations.cc:118-339
+//   Adasum dispatch     ops/adasum/adasum.h:101-140,344-410
+//   FuseResponses       common/controller.cc:793-866
+// Errors become std::logic_error("<op> failed: <text>") exactly as
+// GPUContext::ErrorCheck does (ops/cuda_operations.cc:82-86).
+//
+// The reference's own headers cannot be included here (they pull in Eigen,
+// Boost and FlatBuffers), so the few types the hooks touch are restated in
+// minimal form: DataType, TensorTableEntry (tensor/output pointer, size,
+// dtype, device), Event.
+#ifndef HVD_HIP_ADAPTER_H
+#define HVD_HIP_ADAPTER_H
+
+#include <cstddef>
+#include <cstdint>
+#include <functional>
+#include <map>
+#include <memory>
+#include <queue>
+#include <string>
+#include <unordered_map>
+#include <utility>
+#include <vector>
+
+#include "hvdhip.h"
+
+namespace horovod {
+namespace common {
+
+// common/message.h:30-41
+enum DataType {
+  HOROVOD_UINT8 = 0, HOROVOD_INT8 = 1, HOROVOD_UINT16 = 2, HOROVOD_INT16 = 3, HOROVOD_INT32 = 4,
+  HOROVOD_INT64 = 5, HOROVOD_FLOAT16 = 6, HOROVOD_FLOAT32 = 7, HOROVOD_FLOAT64 = 8, HOROVOD_BOOL = 9
+};
+std::size_t DataType_Size(DataType value);            // common/message.cc:66-92
+const std::string& DataType_Name(DataType value);     // common/message.cc:40-64
+
+typedef void* gpuStream_t;
+
+// The part of TensorTableEntry (common/common.h:341-374) that the hooks read:
+// tensor->data()/size()/dtype(), output->data(), device.
+struct TensorTableEntry {
+  std::string tensor_name;
+  const void* tensor_data = nullptr;
+  void* output_data = nullptr;
+  int64_t num_elements = 0;
+  DataType dtype = HOROVOD_FLOAT32;
+  int device = 0;
+  int64_t tensor_size() const { return num_elements * (int64_t)DataType_Size(dtype); }
+};
+
+// common/common.h:181-189
+struct Event {
+  std::shared_ptr<void*> event;
+  gpuStream_t stream = nullptr;
+};
+
+class GPUContext {
+public:
+  GPUContext();
+  ~GPUContext();
+
+  // One stream per (stream slot, device), created lazily (ops/gpu_operations.cc:30-39).
+  std::vector<std::unordered_map<int, gpuStream_t>> streams;
+
+  void ErrorCheck(std::string op_name, int gpu_result);
+  void RecordEvent(std::queue<std::pair<std::string, Event>>& event_queue, std::string name, gpuStream_t& stream);
+  Event RecordEvent(gpuStream_t& stream);
+  void ReleaseEvent(Event event);
+  // Synchronises every queued event (or polls it when elastic is set, calling
+  // error_check_callback between polls), then recycles it.
+  void WaitForEvents(std::queue<std::pair<std::string, Event>>& event_queue,
+                     const std::function<void()>& error_check_callback = nullptr, bool elastic = false);
+  void ClearEvents(std::queue<std::pair<std::string, Event>>& event_queue);
+  void StreamCreate(gpuStream_t* stream);
+  void StreamSynchronize(gpuStream_t stream);
+  int GetDevice();
+  void SetDevice(int device);
+  void MemcpyAsyncD2D(void* dst, const void* src, size_t count, gpuStream_t stream);
+  void MemcpyAsyncH2D(void* dst, const void* src, size_t count, gpuStream_t stream);
+  void MemcpyAsyncD2H(void* dst, const void* src, size_t count, gpuStream_t stream);
+  void ScaleBufferImpl(const void* fused_input_data, void* buffer_data, int64_t num_elements,
+                       double scale_factor, DataType dtype, gpuStream_t stream);
+};
+
+// The slice of HorovodGlobalState the hooks read (common/global_state.h).
+struct GlobalState {
+  int current_nccl_stream = 0;
+  int num_nccl_streams = 1;
+  bool batch_d2d_memcopies = true;
+  bool enable_async_completion = false;
+  bool elastic_enabled = false;
+  // One fusion buffer per stream slot (common/fusion_buffer_manager.cc:25); owned by the framework.
+  std::vector<void*> fusion_buffer;
+};
+
+class GPUOpContext {
+public:
+  GPUOpContext(GPUContext* context, GlobalState* global_state);
+  void InitGPU(const std::vector<TensorTableEntry>& entries);
+  void InitGPUQueue(const std::vector<TensorTableEntry>& entries);
+  // Records the completion event, waits for the queued events (the reference
+  // hands this to a finalizer thread; here it runs inline), rotates the stream slot.
+  void FinalizeGPUQueue(std::vector<TensorTableEntry>& entries,
+                        const std::function<void()>& error_check_callback = nullptr);
+  std::queue<std::pair<std::string, Event>> event_queue;
+  gpuStream_t* stream = nullptr;
+
+private:
+  GPUContext* gpu_context_;
+  GlobalState* global_state_;
+};
+
+class GPUAllreduce {
+public:
+  GPUAllreduce(GPUContext* context, GlobalState* global_state);
+  ~GPUAllreduce();
+
+  // The op sequence of NCCLAllreduce::Execute (ops/nccl_operations.cc:156-214) with the
+  // collective replaced by a local sum with `peers` (device buffers laid out like the
+  // fusion buffer, or like the single tensor).
+  void Execute(std::vector<TensorTableEntry>& entries, double prescale_factor, double postscale_factor,
+               const std::vector<const void*>& peers);
+
+  void MemcpyInFusionBuffer(const std::vector<TensorTableEntry>& entries, const void*& fused_input_data,
+                            void*& buffer_data, size_t& buffer_len);
+  void MemcpyOutFusionBuffer(const void* buffer_data, std::vector<TensorTableEntry>& entries);
+  void ScaleMemcpyInFusionBuffer(const std::vector<TensorTableEntry>& entries, const void*& fused_input_data,
+                                 void*& buffer_data, size_t& buffer_len, double scale_factor);
+  void ScaleMemcpyOutFusionBuffer(void* buffer_data, size_t buffer_len, double scale_factor,
+                                  std::vector<TensorTableEntry>& entries);
+  void MemcpyEntryInFusionBuffer(const std::vector<TensorTableEntry>& entries, const TensorTableEntry& e,
+                                 void* buffer_data_at_offset);
+  void MemcpyEntryOutFusionBuffer(const std::vector<TensorTableEntry>& entries,
+                                  const void* buffer_data_at_offset, TensorTableEntry& e);
+  void ScaleBuffer(double scale_factor, const std::vector<TensorTableEntry>& entries,
+                   const void* fused_input_data, void* buffer_data, int64_t num_elements);
+
+  size_t cached_plans() const { return plans_.size(); }
+
+private:
+  // Fused tensor sets repeat every step (the reference caches responses,
+  // common/response_cache.cc:126-235): one resident plan per distinct entry list.
+  hvdhip_fusion_plan* PlanFor(const std::vector<TensorTableEntry>& entries);
+  gpuStream_t Stream(const std::vector<TensorTableEntry>& entries);
+
+  GPUContext* gpu_context_;
+  GlobalState* global_state_;
+  GPUOpContext gpu_op_context_;
+  std::map<std::vector<uint64_t>, hvdhip_fusion_plan*> plans_;
+};
+
+// Adasum<Comm>'s dispatch hooks and pairwise reduce, run on the device instead of the
+// host (the reference copies the shard to host first, ops/adasum_gpu_operations.cc:200-211).
+class AdasumGPU {
+public:
+  explicit AdasumGPU(GPUContext* context);
+  ~AdasumGPU();
+  void DispatchComputeDotAndNormSqrds(const void* a, const void* b, DataType horovod_datatype, int count,
+                                      double& dotProduct, double& anormsq, double& bnormsq,
+                                      gpuStream_t stream);
+  void DispatchScaledAdd(DataType horovod_datatype, int count, double acoeff, void* a, double bcoeff,
+                         void* b, gpuStream_t stream);
+  // FusedPairwiseReduceWithComm (ops/adasum/adasum.h:344-410) for one process: per-layer
+  // triples, coefficients and scaled add without leaving the device.  normAndDots, if not
+  // null, receives 3 doubles per layer.
+  void FusedPairwiseReduce(void* a, const void* b, DataType horovod_datatype,
+                           const std::vector<int>& tensor_counts, std::vector<double>* normAndDots,
+                           gpuStream_t stream);
+
+private:
+  GPUContext* gpu_context_;
+  std::map<std::pair<int, std::vector<int>>, hvdhip_adasum_plan*> plans_;
+};
+
+// Controller::FuseResponses (common/controller.cc:793-866) for allreduce responses of one
+// dtype and one pair of scale factors: returns groups of entry indices.
+std::vector<std::vector<int>> FuseResponses(const std::vector<int64_t>& tensor_bytes,
+                                            int64_t fusion_threshold_bytes, bool batch_d2d_memcopies);
+
+}  // namespace common
+}  // namespace horovod
+
+#endif  // HVD_HIP_ADAPTER_H

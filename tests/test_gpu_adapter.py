@@ -1,0 +1,226 @@
+"""The C++ adapter (GPUContext / GPUOpContext / GPUAllreduce hooks / Adasum
+dispatch shaped like the reference's classes) driven on the GPU and compared
+with the oracle's restatement of the same op sequence."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+from oracle_util import F16, F32, F64, I32, U16, NP_OF, SIZE_OF
+
+pytestmark = pytest.mark.gpu
+
+from gpu_util import Arena  # noqa: E402
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def adapter(gpu):
+    lib = ctypes.CDLL(os.path.join(ROOT, "horovod_amd", "lib", "libhvdhip_adapter.so"))
+    lib.hvd_adapter_create.restype = ctypes.c_void_p
+    lib.hvd_adapter_create.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p]
+    lib.hvd_adapter_destroy.argtypes = [ctypes.c_void_p]
+    lib.hvd_adapter_allreduce.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                          ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_double,
+                                          ctypes.c_void_p, ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t]
+    lib.hvd_adapter_state.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
+    lib.hvd_adapter_adasum_pairwise.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                                ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_char_p,
+                                                ctypes.c_size_t]
+    lib.hvd_adapter_adasum_dispatch.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                                ctypes.c_int, ctypes.c_void_p, ctypes.c_double, ctypes.c_double,
+                                                ctypes.c_char_p, ctypes.c_size_t]
+    return lib
+
+
+def _ptrs(values):
+    arr = (ctypes.c_void_p * max(len(values), 1))()
+    for i, v in enumerate(values):
+        arr[i] = v
+    return arr
+
+
+class Harness:
+    def __init__(self, lib, gpu, num_streams=2, batch=True, async_completion=False, elastic=False, fb_bytes=1 << 22):
+        self.lib = lib
+        self.fbs = [gpu.empty(fb_bytes, fill=0xCD) for _ in range(num_streams)]
+        self.h = lib.hvd_adapter_create(num_streams, int(batch), int(async_completion), int(elastic),
+                                        _ptrs([t.data_ptr() for t in self.fbs]))
+
+    def allreduce(self, tensors, outputs, counts, dtype, prescale, postscale, peers=()):
+        err = ctypes.create_string_buffer(512)
+        cnt = (ctypes.c_int64 * len(counts))(*counts)
+        rc = self.lib.hvd_adapter_allreduce(self.h, _ptrs(tensors), _ptrs(outputs), cnt, len(counts), dtype,
+                                            prescale, postscale, _ptrs(list(peers)), len(peers), err, 512)
+        return rc, err.value.decode()
+
+    def state(self):
+        a, b = ctypes.c_int(), ctypes.c_int()
+        self.lib.hvd_adapter_state(self.h, ctypes.byref(a), ctypes.byref(b))
+        return a.value, b.value
+
+    def close(self):
+        self.lib.hvd_adapter_destroy(self.h)
+
+
+def _raw(v):
+    return v.view(np.uint16) if v.dtype == np.float16 else v
+
+
+@pytest.mark.parametrize("batch", [True, False])
+@pytest.mark.parametrize("dtype", [F32, F16])
+def test_execute_fused_matches_the_cpu_op_sequence(gpu, orc, adapter, batch, dtype):
+    """pack -> (prescale) -> sum with two peers -> (postscale) -> unpack, fused entries.
+    batch=False is the per-entry memcpy fallback (HOROVOD_BATCH_D2D_MEMCOPIES=0) with the
+    unpadded layout of ops/gpu_operations.cc:209-222."""
+    rng = np.random.default_rng(1)
+    np_t, es = NP_OF[dtype], SIZE_OF[dtype]
+    counts = [5, 1000, 3, 70001, 256, 1]
+    src, dst = Arena(1 << 20), Arena(1 << 20, fill=0x5A)
+    so, do, vals = [], [], []
+    for c in counts:
+        so.append(src.alloc(c * es)), do.append(dst.alloc(c * es))
+        v = (rng.standard_normal(c) * 1e-2).astype(np_t)
+        src.host[so[-1]:so[-1] + c * es] = v.view(np.uint8)
+        vals.append(v)
+    src.upload(), dst.upload()
+    # peers are laid out like the fusion buffer of the chosen mode
+    offs = orc.padded_offsets([c * es for c in counts]) if batch else np.concatenate([[0], np.cumsum([c * es for c in counts])])
+    peer_vals = [[(rng.standard_normal(c) * 1e-2).astype(np_t) for c in counts] for _ in range(2)]
+    peers = []
+    for pv in peer_vals:
+        img = np.zeros(int(offs[-1]) + 64, np.uint8)
+        for o, v in zip(offs, pv):
+            img[o:o + v.nbytes] = v.view(np.uint8)
+        peers.append(gpu.upload(img))
+    h = Harness(adapter, gpu, num_streams=2, batch=batch)
+    try:
+        for rep in range(3):  # rotates over both stream slots; the plan is built once
+            rc, msg = h.allreduce([src.ptr(o) for o in so], [dst.ptr(o) for o in do], counts, dtype, 0.125, 0.5,
+                                  [p.data_ptr() for p in peers])
+            assert rc == 0, msg
+        out = dst.download()
+        for i, (c, v) in enumerate(zip(counts, vals)):
+            w = orc.scale_buffer(_raw(v), 0.125, dtype)
+            for pv in peer_vals:
+                w = orc.sum(_raw(pv[i]), w, dtype)
+            w = orc.scale_buffer(w, 0.5, dtype)
+            assert np.array_equal(out[do[i]:do[i] + c * es], w.view(np.uint8)), "entry %d" % i
+        cur, plans = h.state()
+        assert cur == 3 % 2  # current_nccl_stream rotated after every op (ops/gpu_operations.cc:101-103)
+        assert plans == (1 if batch else 0)
+    finally:
+        h.close()
+
+
+@pytest.mark.parametrize("prescale,postscale", [(0.125, 1.0), (1.0, 1.0), (1.0, 0.25)])
+def test_execute_single_entry_goes_tensor_to_output(gpu, orc, adapter, prescale, postscale):
+    # ops/nccl_operations.cc:176-186: one entry, no fusion buffer; the fusion buffers stay untouched
+    rng = np.random.default_rng(2)
+    v = rng.standard_normal(100003).astype(np.float32)
+    p = rng.standard_normal(100003).astype(np.float32)
+    d_v, d_o, d_p = gpu.upload(v), gpu.empty(v.nbytes, fill=0), gpu.upload(p)
+    h = Harness(adapter, gpu, num_streams=1)
+    try:
+        rc, msg = h.allreduce([d_v.data_ptr()], [d_o.data_ptr()], [v.size], F32, prescale, postscale, [d_p.data_ptr()])
+        assert rc == 0, msg
+        w = v if prescale == 1.0 else orc.scale_buffer(v, prescale, F32)
+        w = orc.sum(p, w, F32)
+        w = w if postscale == 1.0 else orc.scale_buffer(w, postscale, F32)
+        assert np.array_equal(gpu.download(d_o, np.float32).view(np.uint32), w.view(np.uint32))
+        assert np.array_equal(gpu.download(d_v, np.float32), v)  # input untouched
+        assert np.all(gpu.download(h.fbs[0]) == 0xCD)
+    finally:
+        h.close()
+
+
+def test_async_completion_and_elastic_polling_paths(gpu, orc, adapter):
+    rng = np.random.default_rng(3)
+    v = [rng.standard_normal(5000).astype(np.float32) for _ in range(3)]
+    d_v = [gpu.upload(x) for x in v]
+    d_o = [gpu.empty(x.nbytes, fill=0) for x in v]
+    for async_c, elastic in ((True, False), (False, True)):
+        h = Harness(adapter, gpu, num_streams=1, async_completion=async_c, elastic=elastic)
+        try:
+            rc, msg = h.allreduce([t.data_ptr() for t in d_v], [t.data_ptr() for t in d_o], [5000] * 3, F32, 0.5, 1.0)
+            assert rc == 0, msg
+            import torch
+            torch.cuda.synchronize()
+            for x, o in zip(v, d_o):
+                assert np.array_equal(o.cpu().numpy().view(np.float32), orc.scale_buffer(x, 0.5, F32))
+        finally:
+            h.close()
+
+
+def test_errors_surface_as_logic_error_text(gpu, adapter):
+    t = gpu.empty(4096)
+    h = Harness(adapter, gpu, num_streams=1)
+    try:
+        # UINT16 cannot be scaled: the reference throws "Type uint16 not supported by ..." (cuda_kernels.cu:317-319)
+        rc, msg = h.allreduce([t.data_ptr(), t.data_ptr() + 64], [t.data_ptr() + 128, t.data_ptr() + 256], [8, 8],
+                              U16, 0.5, 1.0)
+        assert rc == -1 and "Type uint16 not supported by BatchedScaledD2DMemcpyCudaImpl" in msg
+        rc, msg = h.allreduce([t.data_ptr()], [t.data_ptr() + 128], [8], U16, 0.5, 1.0)
+        assert rc == -1 and "not supported by ScaleBufferCudaImpl" in msg
+        # a HIP-level failure keeps the "<op> failed: <text>" shape of GPUContext::ErrorCheck
+        rc, msg = h.allreduce([t.data_ptr() + 2, t.data_ptr()], [t.data_ptr() + 128, t.data_ptr() + 256], [8, 8],
+                              F32, 1.0, 1.0)
+        assert rc == -1 and " failed: " in msg
+    finally:
+        h.close()
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, F64])
+def test_adasum_pairwise_on_device(gpu, orc, adapter, dtype):
+    rng = np.random.default_rng(4)
+    np_t = NP_OF[dtype]
+    counts = [1000, 0, 33333, 7]
+    a = rng.standard_normal(sum(counts)).astype(np_t)
+    b = (0.3 * a.astype(np.float64) + rng.standard_normal(sum(counts))).astype(np_t)
+    d_a, d_b = gpu.upload(a), gpu.upload(b)
+    h = Harness(adapter, gpu, num_streams=1)
+    try:
+        nd = np.zeros(3 * len(counts))
+        cnt = (ctypes.c_int * len(counts))(*counts)
+        err = ctypes.create_string_buffer(512)
+        for _ in range(2):
+            d_a = gpu.upload(a)
+            rc = adapter.hvd_adapter_adasum_pairwise(h.h, d_a.data_ptr(), d_b.data_ptr(), dtype, cnt, len(counts),
+                                                     nd.ctypes.data, err, 512)
+            assert rc == 0, err.value
+        want, nd_w, _ = orc.adasum_pairwise(_raw(a), _raw(b), counts, dtype)
+        assert np.allclose(nd, nd_w, rtol=1e-11, atol=1e-300)
+        got = gpu.download(d_a, np.uint16 if dtype == F16 else np_t)
+        if dtype == F16:
+            assert np.array_equal(got, want)
+        elif dtype == F32:
+            assert np.all(np.abs(got - want) <= np.spacing(np.abs(want)))
+        else:
+            assert np.all(np.abs(got - want) <= 1e-11 * (np.abs(a) + np.abs(b)))
+        rc = adapter.hvd_adapter_adasum_pairwise(h.h, d_a.data_ptr(), d_b.data_ptr(), I32, cnt, len(counts),
+                                                 nd.ctypes.data, err, 512)
+        assert rc == -1 and b"Unsupported data type" in err.value
+    finally:
+        h.close()
+
+
+def test_adasum_dispatch_hooks(gpu, orc, adapter):
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal(50001).astype(np.float32)
+    b = rng.standard_normal(50001).astype(np.float32)
+    d_a, d_b = gpu.upload(a), gpu.upload(b)
+    h = Harness(adapter, gpu, num_streams=1)
+    try:
+        out3 = np.zeros(3)
+        err = ctypes.create_string_buffer(512)
+        rc = adapter.hvd_adapter_adasum_dispatch(h.h, d_a.data_ptr(), d_b.data_ptr(), F32, a.size, out3.ctypes.data,
+                                                 0.75, 1.25, err, 512)
+        assert rc == 0, err.value
+        assert np.allclose(out3, orc.adasum_dot_norms(a, b, F32), rtol=1e-12)
+        want = orc.adasum_scaled_add(a, b, 0.75, 1.25, F32)
+        got = gpu.download(d_a, np.float32)
+        assert np.all(np.abs(got - want) <= np.spacing(np.abs(want)))
+    finally:
+        h.close()
