@@ -64,6 +64,7 @@ uint32_t chunk_bytes(Family f) {
   if (forced) return forced;
   switch (f) {
   case Family::kXfer: return kXferChunkBytes;
+  case Family::kXferNarrowing: return kXferNarrowingChunkBytes;
   case Family::kReduce: return kReduceChunkBytes;
   default: return kAdasumChunkBytes;
   }

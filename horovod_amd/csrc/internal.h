@@ -59,8 +59,9 @@ constexpr int kWG = 256;
 // of many small workgroups hides latency better than unrolling inside one.
 // The Adasum reduction pays a workgroup-wide tree per chunk and prefers 16 KiB.
 // HVDHIP_CHUNK_BYTES (a multiple of 4096) overrides all three, for tuning.
-enum class Family { kXfer, kReduce, kAdasum };
+enum class Family { kXfer, kXferNarrowing, kReduce, kAdasum };
 constexpr uint32_t kXferChunkBytes = 4096;
+constexpr uint32_t kXferNarrowingChunkBytes = 8192;  // fp32 -> fp16 pack: 8-byte stores per lane
 constexpr uint32_t kReduceChunkBytes = 4096;
 constexpr uint32_t kAdasumChunkBytes = 16384;
 uint32_t chunk_bytes(Family f);

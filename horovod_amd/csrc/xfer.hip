@@ -323,7 +323,9 @@ struct hvdhip_fusion_plan {
   int buffer_dtype = 0;
   int64_t buffer_len = 0;
   std::vector<int64_t> offsets;
-  DevTables tables;
+  DevTables tables;       // pack (and unpack, when not converting)
+  DevTables unpack_tables;  // converting plans only: unpack prefers smaller chunks than pack
+  bool converting = false;
 };
 
 extern "C" {
@@ -424,7 +426,17 @@ int hvdhip_fusion_plan_create(const void* const* tensors, void* const* outputs,
   p->buffer_dtype = buffer_dtype;
   p->buffer_len = off;
   p->offsets.swap(offsets);
-  int rc = build_tables(segs, chunk_bytes(Family::kXfer) / (uint32_t)std::max(ts, bs), (uint32_t)ts, (uint32_t)bs, &p->tables);
+  p->converting = buffer_dtype != tensor_dtype;
+  // Chunks are sized on the wider (tensor) side.  The narrowing pack stores only 8 bytes per
+  // lane and access and streams best with 8 KiB of fp32 per workgroup; the widening unpack and
+  // every same-width transfer with 4 KiB.
+  const uint32_t wide = (uint32_t)std::max(ts, bs);
+  const uint32_t pack_bytes = p->converting ? chunk_bytes(Family::kXferNarrowing) : chunk_bytes(Family::kXfer);
+  int rc = build_tables(segs, pack_bytes / wide, (uint32_t)ts, (uint32_t)bs, &p->tables);
+  if (rc == 0 && p->converting) {
+    rc = build_tables(segs, chunk_bytes(Family::kXfer) / wide, (uint32_t)ts, (uint32_t)bs, &p->unpack_tables);
+    if (rc) free_tables(&p->tables);
+  }
   if (rc) {
     delete p;
     return rc;
@@ -438,7 +450,9 @@ int hvdhip_fusion_plan_destroy(hvdhip_fusion_plan* plan) {
   // Queued kernels may still read the tables.
   HVDHIP_CHECK(hipDeviceSynchronize());
   int rc = free_tables(&plan->tables);
+  int rc2 = free_tables(&plan->unpack_tables);
   delete plan;
+  if (rc == 0) rc = rc2;
   return rc ? rc : ok();
 }
 
@@ -488,7 +502,7 @@ int hvdhip_fusion_unpack(hvdhip_fusion_plan* plan, const void* fusion_buffer,
   const uint64_t base = (uint64_t)(uintptr_t)fusion_buffer;
   int rc;
   if (plan->buffer_dtype != plan->tensor_dtype) {
-    rc = launch_xfer<UnpackF16F32, kUnpack>(plan->tables, base, {(float)scale_factor}, s);
+    rc = launch_xfer<UnpackF16F32, kUnpack>(plan->unpack_tables, base, {(float)scale_factor}, s);
   } else {
     if (scale_factor != 1.0 && !scalable(plan->tensor_dtype))
       return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE, "dtype %d cannot be scaled", plan->tensor_dtype);
