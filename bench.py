@@ -157,6 +157,45 @@ def cpu_baseline_stress(counts, host, budget_s=12.0):
                       % (reps, dt, os.cpu_count())}
 
 
+def per_tensor_comparator(counts, src, dst, reps=20):
+    """The fusion stress step through the C++ adapter's GPUAllreduce::Execute twice: with the
+    offset-table kernels, and with one hipMemcpyAsync per tensor each way plus a whole-buffer
+    ScaleBuffer (HOROVOD_BATCH_D2D_MEMCOPIES=0, what Horovod does on ROCm today,
+    ops/gpu_operations.cc:209-222,230-235,327-332).  Both include the op's completion wait."""
+    import ctypes
+    import torch
+    lib = ctypes.CDLL(os.path.join(ROOT, "horovod_amd", "lib", "libhvdhip_adapter.so"))
+    lib.hvd_adapter_create.restype = ctypes.c_void_p
+    lib.hvd_adapter_create.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p]
+    lib.hvd_adapter_destroy.argtypes = [ctypes.c_void_p]
+    lib.hvd_adapter_allreduce.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                          ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_double,
+                                          ctypes.c_void_p, ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t]
+    n = len(counts)
+    fb = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
+    fbs = (ctypes.c_void_p * 1)(fb.data_ptr())
+    tp = (ctypes.c_void_p * n)(*src.ptrs)
+    op = (ctypes.c_void_p * n)(*dst.ptrs)
+    cnt = (ctypes.c_int64 * n)(*counts)
+    err = ctypes.create_string_buffer(512)
+    out = {}
+    for name, batch in (("offset_table_kernels_ms", 1), ("per_tensor_copies_ms", 0)):
+        h = lib.hvd_adapter_create(1, batch, 0, 0, fbs)
+        for _ in range(3):
+            rc = lib.hvd_adapter_allreduce(h, tp, op, cnt, n, 7, 0.125, 1.0, None, 0, err, 512)
+            if rc != 0:
+                raise RuntimeError(err.value.decode())
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            lib.hvd_adapter_allreduce(h, tp, op, cnt, n, 7, 0.125, 1.0, None, 0, err, 512)
+        torch.cuda.synchronize()
+        out[name] = round((time.perf_counter() - t0) / reps * 1e3, 4)
+        lib.hvd_adapter_destroy(h)
+    out["speedup"] = round(out["per_tensor_copies_ms"] / out["offset_table_kernels_ms"], 1)
+    return out
+
+
 def extras(steps, warmup):
     """The other pipelines, each as algorithmic GB/s and fraction of the HBM peak."""
     import torch
@@ -326,12 +365,14 @@ def main():
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline_stress(counts, host)
+    comparator = None if args.no_extra else per_tensor_comparator(counts, sets[0][0], sets[0][1])
     for p in plans:
         p.destroy()
     del fbs, sets
     torch.cuda.empty_cache()
     if not args.no_extra:
         result["extra"] = extras(args.steps, args.warmup)
+        result["extra"]["fusion_stress_execute_vs_per_tensor_copies"] = comparator
     print(json.dumps(result))
 
 

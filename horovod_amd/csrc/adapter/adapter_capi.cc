@@ -72,6 +72,22 @@ int hvd_adapter_allreduce(void* handle, const void* const* tensors, void* const*
   }
 }
 
+// Switches the timeline hooks on or off.
+void hvd_adapter_set_timeline(void* handle, int on) {
+  static_cast<Harness*>(handle)->state.timeline_initialized = on != 0;
+}
+
+// Copies the activity names waited for so far, separated by ',', and clears them.
+int hvd_adapter_timeline(void* handle, char* out, size_t outlen) {
+  Harness* h = static_cast<Harness*>(handle);
+  std::string s;
+  for (auto& a : h->state.timeline_activities) s += (s.empty() ? "" : ",") + a;
+  h->state.timeline_activities.clear();
+  std::strncpy(out, s.c_str(), outlen - 1);
+  out[outlen - 1] = 0;
+  return 0;
+}
+
 int hvd_adapter_state(void* handle, int* current_stream, int* cached_plans) {
   Harness* h = static_cast<Harness*>(handle);
   *current_stream = h->state.current_nccl_stream;

@@ -60,8 +60,10 @@ void GPUContext::ReleaseEvent(Event event) {
 }
 
 void GPUContext::WaitForEvents(std::queue<std::pair<std::string, Event>>& event_queue,
-                               const std::function<void()>& error_check_callback, bool elastic) {
+                               const std::function<void()>& error_check_callback, bool elastic,
+                               std::vector<std::string>* timeline_activities) {
   while (!event_queue.empty()) {
+    std::string name = event_queue.front().first;
     Event event = event_queue.front().second;
     event_queue.pop();
     if (elastic) {
@@ -79,6 +81,8 @@ void GPUContext::WaitForEvents(std::queue<std::pair<std::string, Event>>& event_
       if (rc != 0) throw std::logic_error(std::string("hipEventSynchronize failed: ") + hvdhip_error_string(rc));
       if (error_check_callback) error_check_callback();
     }
+    // timeline.ActivityStartAll(entries, name) ... ActivityEndAll(entries) bracket the wait
+    if (name != "" && timeline_activities) timeline_activities->push_back(name);
     ErrorCheck("ReleaseGpuEvent", hvdhip_event_release(event.stream, *event.event));
   }
 }
@@ -135,14 +139,17 @@ void GPUOpContext::InitGPU(const std::vector<TensorTableEntry>& entries) {
 void GPUOpContext::InitGPUQueue(const std::vector<TensorTableEntry>& entries) {
   event_queue = std::queue<std::pair<std::string, Event>>();
   stream = &gpu_context_->streams[(size_t)global_state_->current_nccl_stream][entries[0].device];
+  if (global_state_->timeline_initialized) gpu_context_->RecordEvent(event_queue, QUEUE, *stream);
 }
 
 void GPUOpContext::FinalizeGPUQueue(std::vector<TensorTableEntry>& entries,
                                     const std::function<void()>& error_check_callback) {
   if (!global_state_->enable_async_completion) gpu_context_->RecordEvent(event_queue, "", *stream);
   gpu_context_->SetDevice(entries[0].device);
-  if (!global_state_->enable_async_completion) {
-    gpu_context_->WaitForEvents(event_queue, error_check_callback, global_state_->elastic_enabled);
+  if (!global_state_->enable_async_completion || global_state_->timeline_initialized) {
+    // with the timeline on, events are waited for on the host for accurate timings (ops/gpu_operations.cc:77-80)
+    gpu_context_->WaitForEvents(event_queue, error_check_callback, global_state_->elastic_enabled,
+                                &global_state_->timeline_activities);
   } else {
     gpu_context_->ClearEvents(event_queue);
     Event event = gpu_context_->RecordEvent(*stream);  // handed to the framework in Status.event
@@ -272,8 +279,10 @@ void GPUAllreduce::Execute(std::vector<TensorTableEntry>& entries, double presca
   const void* fused_input_data;
   void* buffer_data;
   size_t buffer_len;
+  const bool timeline = global_state_->timeline_initialized;
   if (entries.size() > 1) {
     ScaleMemcpyInFusionBuffer(entries, fused_input_data, buffer_data, buffer_len, prescale_factor);
+    if (timeline) gpu_context_->RecordEvent(gpu_op_context_.event_queue, MEMCPY_IN_FUSION_BUFFER, *gpu_op_context_.stream);
   } else {
     // ops/nccl_operations.cc:176-186: no fusion buffer, tensor -> output
     fused_input_data = first_entry.tensor_data;
@@ -299,8 +308,10 @@ void GPUAllreduce::Execute(std::vector<TensorTableEntry>& entries, double presca
       done += (size_t)k;
     }
   }
+  if (timeline) gpu_context_->RecordEvent(gpu_op_context_.event_queue, NCCL_ALLREDUCE, *gpu_op_context_.stream);
   if (entries.size() > 1) {
     ScaleMemcpyOutFusionBuffer(buffer_data, buffer_len, postscale_factor, entries);
+    if (timeline) gpu_context_->RecordEvent(gpu_op_context_.event_queue, MEMCPY_OUT_FUSION_BUFFER, *gpu_op_context_.stream);
   } else if (postscale_factor != 1.0) {
     ScaleBuffer(postscale_factor, entries, buffer_data, buffer_data, first_entry.num_elements);
   }

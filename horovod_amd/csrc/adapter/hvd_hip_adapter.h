@@ -45,6 +45,12 @@ const std::string& DataType_Name(DataType value);     // common/message.cc:40-64
 
 typedef void* gpuStream_t;
 
+// Activity names of the stages on this path, common/common.h:73-105.
+#define QUEUE "QUEUE"
+#define MEMCPY_IN_FUSION_BUFFER "MEMCPY_IN_FUSION_BUFFER"
+#define MEMCPY_OUT_FUSION_BUFFER "MEMCPY_OUT_FUSION_BUFFER"
+#define NCCL_ALLREDUCE "NCCL_ALLREDUCE"
+
 // The part of TensorTableEntry (common/common.h:341-374) that the hooks read:
 // tensor->data()/size()/dtype(), output->data(), device.
 struct TensorTableEntry {
@@ -78,7 +84,8 @@ public:
   // Synchronises every queued event (or polls it when elastic is set, calling
   // error_check_callback between polls), then recycles it.
   void WaitForEvents(std::queue<std::pair<std::string, Event>>& event_queue,
-                     const std::function<void()>& error_check_callback = nullptr, bool elastic = false);
+                     const std::function<void()>& error_check_callback = nullptr, bool elastic = false,
+                     std::vector<std::string>* timeline_activities = nullptr);
   void ClearEvents(std::queue<std::pair<std::string, Event>>& event_queue);
   void StreamCreate(gpuStream_t* stream);
   void StreamSynchronize(gpuStream_t stream);
@@ -98,6 +105,11 @@ struct GlobalState {
   bool batch_d2d_memcopies = true;
   bool enable_async_completion = false;
   bool elastic_enabled = false;
+  // Timeline::Initialized(): when set, the ops enqueue a named event after every stage
+  // (ops/nccl_operations.cc:173-175,195-197,203-205) and the completed activity names are
+  // appended to timeline_activities as the events are waited for.
+  bool timeline_initialized = false;
+  std::vector<std::string> timeline_activities;
   // One fusion buffer per stream slot (common/fusion_buffer_manager.cc:25); owned by the framework.
   std::vector<void*> fusion_buffer;
 };

@@ -154,6 +154,38 @@ def test_async_completion_and_elastic_polling_paths(gpu, orc, adapter):
             h.close()
 
 
+def test_timeline_hooks_record_an_event_after_every_stage(gpu, orc, adapter):
+    # ops/nccl_operations.cc:173-175,195-197,203-205 and ops/gpu_operations.cc:45-47
+    rng = np.random.default_rng(6)
+    v = [rng.standard_normal(4000).astype(np.float32) for _ in range(2)]
+    d_v = [gpu.upload(x) for x in v]
+    d_o = [gpu.empty(x.nbytes, fill=0) for x in v]
+    h = Harness(adapter, gpu, num_streams=1, async_completion=True)
+    try:
+        adapter.hvd_adapter_set_timeline.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        adapter.hvd_adapter_timeline.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]
+        adapter.hvd_adapter_set_timeline(h.h, 1)
+        rc, msg = h.allreduce([t.data_ptr() for t in d_v], [t.data_ptr() for t in d_o], [4000] * 2, F32, 0.5, 1.0)
+        assert rc == 0, msg
+        out = ctypes.create_string_buffer(512)
+        adapter.hvd_adapter_timeline(h.h, out, 512)
+        assert out.value.decode().split(",") == ["QUEUE", "MEMCPY_IN_FUSION_BUFFER", "NCCL_ALLREDUCE",
+                                                 "MEMCPY_OUT_FUSION_BUFFER"]
+        # single entry: no fusion-buffer stages
+        rc, msg = h.allreduce([d_v[0].data_ptr()], [d_o[0].data_ptr()], [4000], F32, 0.5, 1.0)
+        adapter.hvd_adapter_timeline(h.h, out, 512)
+        assert out.value.decode().split(",") == ["QUEUE", "NCCL_ALLREDUCE"]
+        adapter.hvd_adapter_set_timeline(h.h, 0)
+        rc, msg = h.allreduce([t.data_ptr() for t in d_v], [t.data_ptr() for t in d_o], [4000] * 2, F32, 0.5, 1.0)
+        adapter.hvd_adapter_timeline(h.h, out, 512)
+        assert out.value == b""
+        import torch
+        torch.cuda.synchronize()
+        assert np.array_equal(d_o[1].cpu().numpy().view(np.float32), orc.scale_buffer(v[1], 0.5, F32))
+    finally:
+        h.close()
+
+
 def test_errors_surface_as_logic_error_text(gpu, adapter):
     t = gpu.empty(4096)
     h = Harness(adapter, gpu, num_streams=1)
