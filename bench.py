@@ -43,8 +43,11 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--kernel-only", action="store_true",
-                    help="only launch the dominant kernel (for rocprofv3 runs)")
+    ap.add_argument("--kernel-only", nargs="?", const="pack", default=None,
+                    choices=["pack", "reduce", "adasum"],
+                    help="only launch one kernel family (for rocprofv3 runs): the scaled pack of the headline "
+                         "workload (default), the fp32 reduce-sum of a 64 MiB buffer with one peer, or the "
+                         "Adasum combine of 2 x 2^25 fp32 in 64 layers")
     ap.add_argument("--calibrate", action="store_true",
                     help="only launch a plain 256 MiB device copy (scales rocprofv3 byte counters)")
     ap.add_argument("--replicas", type=int, default=8,
@@ -315,6 +318,24 @@ def main():
         torch.cuda.synchronize()
         for _ in range(args.warmup + args.steps):
             H.batched_d2d_memcpy([b.data_ptr()], [a.data_ptr()], [n], stream)
+        stream.synchronize()
+        return
+
+    if args.kernel_only in ("reduce", "adasum"):
+        from horovod_amd import AdasumPlan, host as H, workloads as W
+        g = torch.Generator(device="cuda")
+        g.manual_seed(7)
+        n = (64 << 20) // 4 if args.kernel_only == "reduce" else 1 << 25
+        pairs = [(torch.randn(n, generator=g, device="cuda"), torch.randn(n, generator=g, device="cuda"))
+                 for _ in range(4)]
+        plan = AdasumPlan(W.adasum_layer_counts(n, 64, seed=13), F32) if args.kernel_only == "adasum" else None
+        torch.cuda.synchronize()
+        for i in range(args.warmup + args.steps):
+            a, b = pairs[i % 4]
+            if plan is None:
+                H.reduce_sum(a.data_ptr(), b.data_ptr(), n, F32, stream)
+            else:
+                plan.combine(a.data_ptr(), b.data_ptr(), stream)
         stream.synchronize()
         return
 
