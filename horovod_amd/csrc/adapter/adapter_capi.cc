@@ -131,6 +131,54 @@ int hvd_adapter_adasum_dispatch(void* handle, void* a, void* b, int dtype, int c
   }
 }
 
+// Simulates the fusion-buffer side of a fused allgather over `global_size` ranks on one
+// device: every rank packs its entries (tensors[rank * n + ec], sizes[ec * global_size + rank]
+// elements) into the shared buffer at its displacement -- which stands in for the collective --
+// and then rank 0's outputs are unpacked.  outputs[ec] must hold the sum over ranks.
+int hvd_adapter_allgather(void* handle, const void* const* tensors, void* const* outputs, const int64_t* sizes,
+                          int n, int global_size, int dtype, char* err, size_t errlen) {
+  Harness* h = static_cast<Harness*>(handle);
+  try {
+    GPUAllgather op(&h->context, &h->state);
+    const int es = (int)DataType_Size((DataType)dtype);
+    std::vector<int> recvcounts((size_t)global_size, 0), displ((size_t)global_size, 0);
+    std::vector<std::vector<int64_t>> csz((size_t)n, std::vector<int64_t>((size_t)global_size)),
+        cof((size_t)n, std::vector<int64_t>((size_t)global_size));
+    std::vector<int64_t*> csz_p, cof_p;
+    for (int ec = 0; ec < n; ++ec) {
+      for (int rc = 0; rc < global_size; ++rc) {
+        csz[(size_t)ec][(size_t)rc] = sizes[ec * global_size + rc];
+        recvcounts[(size_t)rc] += (int)sizes[ec * global_size + rc];
+      }
+      csz_p.push_back(csz[(size_t)ec].data());
+      cof_p.push_back(cof[(size_t)ec].data());
+    }
+    int* dp = displ.data();
+    GPUAllgather::SetDisplacements(recvcounts.data(), dp, global_size);
+    int64_t** cofpp = cof_p.data();
+    GPUAllgather::SetEntryComponentOffsets((size_t)n, csz_p.data(), recvcounts.data(), cofpp, global_size);
+    if (h->context.streams.empty()) h->context.streams.resize(1);
+    gpuStream_t& s = h->context.streams[(size_t)h->state.current_nccl_stream][0];
+    if (!s) h->context.StreamCreate(&s);
+    void* buffer_data = nullptr;
+    std::vector<TensorTableEntry> entries((size_t)n);
+    for (int rank = 0; rank < global_size; ++rank) {
+      for (int ec = 0; ec < n; ++ec) {
+        entries[(size_t)ec].tensor_data = tensors[rank * n + ec];
+        entries[(size_t)ec].output_data = outputs[ec];
+        entries[(size_t)ec].num_elements = sizes[ec * global_size + rank];
+        entries[(size_t)ec].dtype = (DataType)dtype;
+      }
+      op.MemcpyInFusionBuffer(entries, displ.data(), rank, es, buffer_data);
+    }
+    op.MemcpyOutFusionBuffer(cof_p.data(), csz_p.data(), buffer_data, es, global_size, entries);
+    h->context.StreamSynchronize(s);
+    return 0;
+  } catch (const std::exception& e) {
+    return report(e, err, errlen);
+  }
+}
+
 int hvd_adapter_fuse(const int64_t* tensor_bytes, int n, int64_t threshold, int batch_d2d_memcopies, int* group_of) {
   std::vector<int64_t> tb(tensor_bytes, tensor_bytes + n);
   auto groups = FuseResponses(tb, threshold, batch_d2d_memcopies != 0);

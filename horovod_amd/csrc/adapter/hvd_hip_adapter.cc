@@ -318,6 +318,70 @@ void GPUAllreduce::Execute(std::vector<TensorTableEntry>& entries, double presca
   gpu_op_context_.FinalizeGPUQueue(entries);
 }
 
+// --------------------------------------------------------------- GPUAllgather
+
+GPUAllgather::GPUAllgather(GPUContext* context, GlobalState* global_state)
+    : gpu_context_(context), global_state_(global_state) {}
+
+void GPUAllgather::SetDisplacements(const int* recvcounts, int*& displcmnts, int global_size) {
+  for (int rc = 0; rc < global_size; ++rc)
+    displcmnts[rc] = rc == 0 ? 0 : displcmnts[rc - 1] + recvcounts[rc - 1];
+}
+
+void GPUAllgather::SetEntryComponentOffsets(size_t num_entries, const int64_t* const* entry_component_sizes,
+                                            const int* recvcounts, int64_t**& entry_component_offsets,
+                                            int global_size) {
+  int64_t rank_displacement = 0;
+  for (int rc = 0; rc < global_size; ++rc) {
+    for (size_t ec = 0; ec < num_entries; ++ec)
+      entry_component_offsets[ec][rc] =
+          ec == 0 ? rank_displacement : entry_component_offsets[ec - 1][rc] + entry_component_sizes[ec - 1][rc];
+    rank_displacement += recvcounts[rc];
+  }
+}
+
+void GPUAllgather::MemcpyInFusionBuffer(const std::vector<TensorTableEntry>& entries, const int* displcmnts,
+                                        int rank, int element_size, void*& buffer_data) {
+  auto& first_entry = entries[0];
+  buffer_data = global_state_->fusion_buffer[(size_t)global_state_->current_nccl_stream];
+  std::vector<void*> out;
+  std::vector<const void*> in;
+  std::vector<size_t> sizes;
+  int64_t offset = (int64_t)displcmnts[rank] * element_size;
+  for (auto& e : entries) {
+    out.push_back((uint8_t*)buffer_data + offset);
+    in.push_back(e.tensor_data);
+    sizes.push_back((size_t)e.tensor_size());
+    offset += e.tensor_size();
+  }
+  gpu_context_->ErrorCheck("hvdhip_batched_d2d_memcpy",
+                           hvdhip_batched_d2d_memcpy(out.data(), in.data(), sizes.data(), (int)sizes.size(),
+                                                     gpu_context_->streams[(size_t)global_state_->current_nccl_stream][first_entry.device]));
+}
+
+void GPUAllgather::MemcpyOutFusionBuffer(const int64_t* const* entry_component_offsets,
+                                         const int64_t* const* entry_component_sizes, const void* buffer_data,
+                                         int element_size, int global_size,
+                                         std::vector<TensorTableEntry>& entries) {
+  std::vector<void*> out;
+  std::vector<const void*> in;
+  std::vector<size_t> sizes;
+  for (size_t ec = 0; ec < entries.size(); ++ec) {
+    int64_t copy_offset = 0;
+    for (int rc = 0; rc < global_size; ++rc) {
+      const int64_t entry_offset = entry_component_offsets[ec][rc] * element_size;
+      const int64_t entry_size = entry_component_sizes[ec][rc] * element_size;
+      out.push_back((uint8_t*)entries[ec].output_data + copy_offset);
+      in.push_back((const uint8_t*)buffer_data + entry_offset);
+      sizes.push_back((size_t)entry_size);
+      copy_offset += entry_size;
+    }
+  }
+  gpu_context_->ErrorCheck("hvdhip_batched_d2d_memcpy",
+                           hvdhip_batched_d2d_memcpy(out.data(), in.data(), sizes.data(), (int)sizes.size(),
+                                                     gpu_context_->streams[(size_t)global_state_->current_nccl_stream][entries[0].device]));
+}
+
 // ------------------------------------------------------------------ AdasumGPU
 
 AdasumGPU::AdasumGPU(GPUContext* context) : gpu_context_(context) {}

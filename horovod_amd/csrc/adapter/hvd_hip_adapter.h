@@ -170,6 +170,31 @@ private:
   std::map<std::vector<uint64_t>, hvdhip_fusion_plan*> plans_;
 };
 
+// The fusion-buffer hooks of the allgather op (ops/collective_operations.cc:200-275,
+// GPU overrides ops/gpu_operations.cc:350-363).  The reference issues one async copy per
+// entry (pack) and per (entry, rank) component (unpack); here each direction is one
+// batched launch.  The collective itself (every rank's slab arriving in the buffer) is
+// outside this class.
+class GPUAllgather {
+public:
+  GPUAllgather(GPUContext* context, GlobalState* global_state);
+  // AllgatherOp::SetDisplacements
+  static void SetDisplacements(const int* recvcounts, int*& displcmnts, int global_size);
+  // AllgatherOp::SetEntryComponentOffsets; the matrices are [entry][rank]
+  static void SetEntryComponentOffsets(size_t num_entries, const int64_t* const* entry_component_sizes,
+                                       const int* recvcounts, int64_t**& entry_component_offsets,
+                                       int global_size);
+  void MemcpyInFusionBuffer(const std::vector<TensorTableEntry>& entries, const int* displcmnts, int rank,
+                            int element_size, void*& buffer_data);
+  void MemcpyOutFusionBuffer(const int64_t* const* entry_component_offsets,
+                             const int64_t* const* entry_component_sizes, const void* buffer_data,
+                             int element_size, int global_size, std::vector<TensorTableEntry>& entries);
+
+private:
+  GPUContext* gpu_context_;
+  GlobalState* global_state_;
+};
+
 // Adasum<Comm>'s dispatch hooks and pairwise reduce, run on the device instead of the
 // host (the reference copies the shard to host first, ops/adasum_gpu_operations.cc:200-211).
 class AdasumGPU {

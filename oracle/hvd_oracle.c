@@ -30,6 +30,8 @@
  *       (test/parallel/test_adasum_tensorflow.py:29-44) and the algebraic
  *       invariants of test/parallel/test_adasum_pytorch.py:46-211.
  *   orc_fuse_responses               hand-computed cases + brute force.
+ *   orc_allgather_*                  closed form: every output equals the
+ *       concatenation over ranks of that entry's per-rank tensor.
  */
 #include <float.h>
 #include <immintrin.h>
@@ -547,4 +549,64 @@ int orc_fuse_responses(const int64_t* tensor_bytes, const int* key, int n, int64
     }
   }
   return ngroups;
+}
+
+/* ------------------------------------------------------------------ */
+/* Allgather fusion buffer                                            */
+/* ------------------------------------------------------------------ */
+
+/* AllgatherOp::SetDisplacements, ops/collective_operations.cc:200-209:
+ * exclusive prefix sum of the per-rank element counts. */
+void orc_allgather_displacements(const int* recvcounts, int* displcmnts, int global_size) {
+  int acc = 0;
+  for (int rc = 0; rc < global_size; ++rc) {
+    displcmnts[rc] = acc;
+    acc += recvcounts[rc];
+  }
+}
+
+/* AllgatherOp::SetEntryComponentOffsets, ops/collective_operations.cc:211-232.
+ * sizes and offsets are row-major [entry][rank] element counts: inside rank
+ * rc's slab (which starts at the sum of the earlier ranks' recvcounts) the
+ * entries follow one another. */
+void orc_allgather_component_offsets(const int64_t* sizes, int nentries, int global_size,
+                                     const int* recvcounts, int64_t* offsets) {
+  int64_t rank_displacement = 0;
+  for (int rc = 0; rc < global_size; ++rc) {
+    for (int ec = 0; ec < nentries; ++ec) {
+      if (ec == 0)
+        offsets[ec * global_size + rc] = rank_displacement;
+      else
+        offsets[ec * global_size + rc] =
+            offsets[(ec - 1) * global_size + rc] + sizes[(ec - 1) * global_size + rc];
+    }
+    rank_displacement += recvcounts[rc];
+  }
+}
+
+/* AllgatherOp::MemcpyInFusionBuffer, ops/collective_operations.cc:234-253:
+ * this rank's entries go, unpadded, to its displacement in the buffer. */
+void orc_allgather_pack(const void* const* tensors, const int64_t* nbytes, int nentries,
+                        const int* displcmnts, int rank, int element_size, void* buf) {
+  int64_t off = (int64_t)displcmnts[rank] * element_size;
+  for (int i = 0; i < nentries; ++i) {
+    memcpy((uint8_t*)buf + off, tensors[i], (size_t)nbytes[i]);
+    off += nbytes[i];
+  }
+}
+
+/* AllgatherOp::MemcpyOutFusionBuffer, ops/collective_operations.cc:255-275:
+ * output ec is the concatenation over ranks of that entry's component. */
+void orc_allgather_unpack(const int64_t* offsets, const int64_t* sizes, int nentries,
+                          int global_size, const void* buf, int element_size,
+                          void* const* outputs) {
+  for (int ec = 0; ec < nentries; ++ec) {
+    int64_t copy_offset = 0;
+    for (int rc = 0; rc < global_size; ++rc) {
+      int64_t eo = offsets[ec * global_size + rc] * element_size;
+      int64_t es = sizes[ec * global_size + rc] * element_size;
+      memcpy((uint8_t*)outputs[ec] + copy_offset, (const uint8_t*)buf + eo, (size_t)es);
+      copy_offset += es;
+    }
+  }
 }

@@ -193,6 +193,28 @@ class Oracle:
             raise ValueError("dtype")
         return out, nd, co
 
+    # ---- allgather fusion ----
+    def allgather(self, per_rank_tensors, dtype):
+        """per_rank_tensors[rank][entry] -> list of outputs (one per entry), via the oracle's
+        displacement / offset / pack / unpack restatement, every rank packing into one buffer."""
+        size, n = len(per_rank_tensors), len(per_rank_tensors[0])
+        es = SIZE_OF[dtype]
+        sizes = np.array([[per_rank_tensors[rc][ec].size for rc in range(size)] for ec in range(n)], np.int64)
+        recv = np.array([int(sizes[:, rc].sum()) for rc in range(size)], np.int32)
+        displ = np.zeros(size, np.int32)
+        self.lib.orc_allgather_displacements(_p(recv), _p(displ), c_int(size))
+        offs = np.zeros((n, size), np.int64)
+        self.lib.orc_allgather_component_offsets(_p(sizes), c_int(n), c_int(size), _p(recv), _p(offs))
+        buf = np.full(int(recv.sum()) * es + 16, 0xEE, np.uint8)
+        for rc in range(size):
+            ts = [np.ascontiguousarray(t) for t in per_rank_tensors[rc]]
+            nb = np.array([t.nbytes for t in ts], np.int64)
+            self.lib.orc_allgather_pack(self._ptrs(ts), _p(nb), c_int(n), _p(displ), c_int(rc), c_int(es), _p(buf))
+        outs = [np.zeros(int(sizes[ec].sum()), per_rank_tensors[0][ec].dtype) for ec in range(n)]
+        self.lib.orc_allgather_unpack(_p(offs), _p(sizes), c_int(n), c_int(size), _p(buf), c_int(es),
+                                      self._ptrs(outs))
+        return outs, displ, offs
+
     # ---- planning ----
     def fusion_threshold(self, proposed, local_size, homogeneous=True):
         return int(self.lib.orc_fusion_threshold(c_int64(proposed), c_int(local_size), c_int(int(homogeneous))))

@@ -186,6 +186,34 @@ def test_timeline_hooks_record_an_event_after_every_stage(gpu, orc, adapter):
         h.close()
 
 
+@pytest.mark.parametrize("dtype", [F32, F16])
+def test_allgather_fusion_buffer_hooks(gpu, orc, adapter, dtype):
+    # every rank's entries packed at its displacement, then unpacked per (entry, rank) component
+    rng = np.random.default_rng(7)
+    np_t, es = NP_OF[dtype], SIZE_OF[dtype]
+    size, n = 4, 5
+    per_rank = [[rng.standard_normal(int(rng.integers(0, 30000))).astype(np_t) for _ in range(n)] for _ in range(size)]
+    want, _, _ = orc.allgather([[_raw(t) for t in r] for r in per_rank], dtype)
+    d_t = [[gpu.upload(t) if t.size else gpu.empty(16) for t in r] for r in per_rank]
+    d_o = [gpu.empty(max(w.nbytes, 16), fill=0x5A) for w in want]
+    sizes = (ctypes.c_int64 * (n * size))(*[per_rank[rc][ec].size for ec in range(n) for rc in range(size)])
+    h = Harness(adapter, gpu, num_streams=1, fb_bytes=1 << 22)
+    try:
+        adapter.hvd_adapter_allgather.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                                  ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_char_p,
+                                                  ctypes.c_size_t]
+        err = ctypes.create_string_buffer(512)
+        rc = adapter.hvd_adapter_allgather(h.h, _ptrs([t.data_ptr() for r in d_t for t in r]),
+                                           _ptrs([t.data_ptr() for t in d_o]), sizes, n, size, dtype, err, 512)
+        assert rc == 0, err.value
+        for ec in range(n):
+            got = gpu.download(d_o[ec])
+            assert np.array_equal(got[:want[ec].nbytes], want[ec].view(np.uint8)), "entry %d" % ec
+            assert np.all(got[want[ec].nbytes:] == 0x5A)
+    finally:
+        h.close()
+
+
 def test_errors_surface_as_logic_error_text(gpu, adapter):
     t = gpu.empty(4096)
     h = Harness(adapter, gpu, num_streams=1)
