@@ -160,6 +160,106 @@ def cpu_baseline_stress(counts, host, budget_s=12.0):
                       % (reps, dt, os.cpu_count())}
 
 
+def cpu_extras(budget_s=2.5):
+    """The CPU oracle on one core over bounded samples of the other pipelines, in the same
+    algorithmic bytes as the GPU figures: the whole ResNet-50 set, one 42-tensor BERT-large cycle
+    (cast and scale fused into the copy, which flatters the CPU), the whole Adasum pair, one
+    GPT-2 XL layer.  Buffers are preallocated and every oracle call works in place."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_util
+    from ctypes import c_double, c_int, c_int64, c_void_p
+    from oracle_util import F16, F32
+    from horovod_amd import workloads as W
+    L = oracle_util.Oracle().lib
+    rng = np.random.default_rng(0)
+    out = {}
+
+    def P(a, off=0):
+        return c_void_p(a.ctypes.data + off)
+
+    def ptrs(arrays):
+        return (c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
+
+    def run(name, fn, nbytes):
+        fn()
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt > budget_s:
+                break
+        out[name] = {"cpu_GB/s": round(nbytes * reps / dt / 1e9, 2), "cores": 1, "reps": reps}
+
+    # ResNet-50: memcpy pack, ScaleBuffer 0.125 in place, sum with one peer, memcpy unpack (7P)
+    counts = [W.numel(s) for s in W.resnet50_shapes()]
+    ts = [(rng.standard_normal(c, dtype=np.float32) * np.float32(1e-3)) for c in counts]
+    outs = [np.empty_like(t) for t in ts]
+    n, k = sum(counts), len(counts)
+    nb = np.array([4 * c for c in counts], np.int64)
+    buf = np.zeros(n, np.float32)
+    peer = rng.standard_normal(n, dtype=np.float32)
+    tp, op = ptrs(ts), ptrs(outs)
+
+    def resnet():
+        L.orc_pack(tp, P(nb), c_int(k), P(buf))
+        L.orc_scale_buffer(P(buf), P(buf), c_int64(n), c_double(0.125), c_int(F32))
+        L.orc_sum(P(peer), P(buf), c_int64(n), c_int(F32))
+        L.orc_unpack(P(buf), op, P(nb), c_int(k))
+
+    run("resnet50_fp32_pack_scale_reduce_unpack", resnet, 7 * 4 * n)
+
+    # BERT-large, one cycle of 42 tensors: fp32 -> fp16 with prescale, 7 peers on 1/8, fp16 -> fp32
+    counts = [W.numel(s) for s in W.bert_large_shapes()][7:49]
+    ts = [(rng.standard_normal(c, dtype=np.float32) * np.float32(1e-4)) for c in counts]
+    outs = [np.empty_like(t) for t in ts]
+    n = sum(counts)
+    hbuf = np.zeros(n, np.uint16)
+    peers = [rng.integers(0, 0x0400, n // 8, dtype=np.uint16) for _ in range(7)]
+
+    def bert():
+        off = 0
+        for t, c in zip(ts, counts):
+            L.orc_scale_cast_f32_to_f16(P(t), P(hbuf, 2 * off), c_int64(c), c_double(0.125))
+            off += c
+        for p in peers:
+            L.orc_float16_sum(P(p), P(hbuf), c_int64(n // 8))
+        off = 0
+        for o, c in zip(outs, counts):
+            L.orc_scale_cast_f16_to_f32(P(hbuf, 2 * off), P(o), c_int64(c), c_double(1.0))
+            off += c
+
+    run("bert_large_fp32_to_fp16_7peers_eighth_chunk", bert, 6 * n + 9 * 2 * (n // 8) + 6 * n)
+
+    # Adasum: the whole pair, in place on a (values stay finite from repetition to repetition)
+    n = 1 << 25
+    lc = np.array(W.adasum_layer_counts(n, 64, seed=13), np.int32)
+    a = rng.standard_normal(n, dtype=np.float32)
+    b = rng.standard_normal(n, dtype=np.float32)
+    nd, co = np.zeros(192), np.zeros(128)
+    run("adasum_fp32_2x32M_64layers",
+        lambda: L.orc_adasum_pairwise(P(a), P(b), c_int(F32), P(lc), c_int(64), P(nd), P(co)), 5 * n * 4)
+
+    # GPT-2 XL: one transformer layer (12 fp16 tensors, 61.5 MB)
+    counts = [W.numel(s) for s in W.gpt2_xl_shapes()][2:14]
+    ts = [rng.integers(0, 0x3c00, c, dtype=np.uint16) for c in counts]
+    outs = [np.empty_like(t) for t in ts]
+    n, k = sum(counts), len(counts)
+    nb = np.array([2 * c for c in counts], np.int64)
+    hbuf = np.zeros(n, np.uint16)
+    peer = rng.integers(0, 0x3c00, n, dtype=np.uint16)
+    tp2, op2 = ptrs(ts), ptrs(outs)
+
+    def gpt2():
+        L.orc_pack(tp2, P(nb), c_int(k), P(hbuf))
+        L.orc_scale_buffer(P(hbuf), P(hbuf), c_int64(n), c_double(0.125), c_int(F16))
+        L.orc_float16_sum(P(peer), P(hbuf), c_int64(n))
+        L.orc_unpack(P(hbuf), op2, P(nb), c_int(k))
+
+    run("gpt2_xl_fp16_two_streams", gpt2, 7 * 2 * n)
+    return out
+
+
 def per_tensor_comparator(counts, src, dst, reps=20):
     """The fusion stress step through the C++ adapter's GPUAllreduce::Execute twice: with the
     offset-table kernels, and with one hipMemcpyAsync per tensor each way plus a whole-buffer
@@ -394,6 +494,10 @@ def main():
     if not args.no_extra:
         result["extra"] = extras(args.steps, args.warmup)
         result["extra"]["fusion_stress_execute_vs_per_tensor_copies"] = comparator
+        if not args.no_cpu:
+            for name, v in cpu_extras().items():
+                result["extra"][name].update({"cpu_GB/s": v["cpu_GB/s"], "cpu_cores": 1,
+                                              "cpu_sample_reps": v["reps"]})
     print(json.dumps(result))
 
 

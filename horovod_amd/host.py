@@ -19,18 +19,23 @@ def _ptr_array(values):
 class Stream:
     """A stream of the library (GPUContext::StreamCreate)."""
 
-    def __init__(self):
-        h = c_void_p()
-        check(lib().hvdhip_stream_create(ctypes.byref(h)), "hvdhip_stream_create")
-        self.handle = h
+    def __init__(self, handle=None):
+        """Creates a stream, or wraps an existing hipStream_t address (not owned)."""
+        self.owned = handle is None
+        if handle is None:
+            h = c_void_p()
+            check(lib().hvdhip_stream_create(ctypes.byref(h)), "hvdhip_stream_create")
+            self.handle = h
+        else:
+            self.handle = c_void_p(handle)
 
     def synchronize(self):
         check(lib().hvdhip_stream_synchronize(self.handle), "hvdhip_stream_synchronize")
 
     def destroy(self):
-        if self.handle is not None:
+        if self.handle is not None and self.owned:
             check(lib().hvdhip_stream_destroy(self.handle), "hvdhip_stream_destroy")
-            self.handle = None
+        self.handle = None
 
 
 class Timer:
