@@ -13,6 +13,13 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+@pytest.fixture(scope="session", autouse=True)
+def _native_libraries():
+    """Loads what is built; builds only if nothing is."""
+    from horovod_amd import build
+    build.ensure_built()
+
+
 @pytest.fixture(scope="session")
 def orc():
     import oracle_util

@@ -1,0 +1,23 @@
+"""The kernels' multi-vector (unrolled) inner loops only run when a workgroup's chunk holds
+more than 1,024 vectors; the default 4 KiB chunks never reach them for transfers.  This runs
+the pack / scale / reduce parity tests once more in a child process with 64 KiB chunks."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_parity_with_64_kib_chunks(gpu):
+    env = dict(os.environ, HVDHIP_CHUNK_BYTES="65536")
+    cmd = [sys.executable, "-m", "pytest", "-q", "-x", "-m", "gpu", "--timeout", "300", "--timeout-method", "thread",
+           os.path.join(ROOT, "tests", "test_gpu_pack.py"), os.path.join(ROOT, "tests", "test_gpu_scale_reduce.py"),
+           os.path.join(ROOT, "tests", "test_gpu_adasum.py"), "-p", "no:cacheprovider"]
+    r = subprocess.run(cmd, cwd=ROOT, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=900)
+    tail = r.stdout.decode(errors="replace")[-3000:]
+    assert r.returncode == 0, tail
+    assert " passed" in tail and "failed" not in tail
