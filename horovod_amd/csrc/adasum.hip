@@ -310,9 +310,10 @@ OneLayerCache& one_layer_cache() {
 }
 constexpr size_t kOneLayerCapacity = 256;
 
+// The caller holds the cache mutex until its work on the plan is queued (and, for the
+// blocking entry point, finished): eviction destroys plans, and plans carry state.
 int one_layer_plan(int count, int dtype, hvdhip_adasum_plan** out) {
   OneLayerCache& c = one_layer_cache();
-  std::lock_guard<std::mutex> g(c.mu);
   for (auto it = c.lru.begin(); it != c.lru.end(); ++it) {
     if ((*it)->total == count && (*it)->dtype == dtype) {
       c.lru.splice(c.lru.begin(), c.lru, it);
@@ -456,6 +457,7 @@ int hvdhip_adasum_dot_and_norm_sqrds(const void* a, const void* b, int dtype, in
   if (!dot || !anormsq || !bnormsq) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "result pointer is NULL");
   if (count < 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "count is negative");
   hvdhip_adasum_plan* p = nullptr;
+  std::lock_guard<std::mutex> g(one_layer_cache().mu);
   int rc = one_layer_plan(count, dtype, &p);
   if (rc) return rc;
   rc = check_vectors(p, a, b);
@@ -475,6 +477,7 @@ int hvdhip_adasum_dispatch_scaled_add(int dtype, int count, double acoeff, void*
                                       double bcoeff, const void* b, void* stream) {
   if (count < 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "count is negative");
   hvdhip_adasum_plan* p = nullptr;
+  std::lock_guard<std::mutex> g(one_layer_cache().mu);
   int rc = one_layer_plan(count, dtype, &p);
   if (rc) return rc;
   rc = check_vectors(p, a, b);

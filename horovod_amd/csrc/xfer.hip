@@ -2,15 +2,18 @@
 // scale and the fp32<->fp16 compression cast fused in, plus the whole-buffer
 // scale.  gfx950 only.
 //
-// One launch moves a whole fused response.  The host describes it with two
-// device-resident tables: one segment per tensor (addresses, fusion-buffer
-// offset, element count) and one chunk per workgroup (segment number, chunk
-// number inside the segment).  A workgroup of four wave64 wavefronts streams
-// its chunk with 16-byte accesses per lane, several loads in flight before
-// the first store; consecutive workgroups touch consecutive addresses of a
-// large tensor, so a single big tensor is spread over all XCDs and HBM stacks
-// while a tiny one costs a single short workgroup.  This is bandwidth-bound
-// byte/element work: no LDS and no matrix cores are involved.
+// One launch moves a whole fused response.  The host describes it with one
+// device-resident table of self-contained 32-byte chunk entries (source,
+// destination, fusion-buffer offset, element count), one per workgroup.  A
+// workgroup of four wave64 wavefronts loads its entry with a single scalar
+// load and streams its chunk with one 16-byte non-temporal access per lane
+// (4 KiB per workgroup: the occupancy of many small workgroups keeps about
+// 8 MiB in flight, which is what HBM latency times bandwidth asks for).
+// Workgroups are dispatched round-robin over the XCDs and consecutive
+// workgroups touch consecutive 4 KiB pieces, so a single big tensor is spread
+// over all XCDs and HBM stacks while a tiny one costs a single short
+// workgroup.  This is bandwidth-bound byte/element work with no reuse: no
+// LDS and no matrix cores are involved.
 //
 // All vector accesses are declared with element alignment only.  gfx950
 // serves multi-dword global accesses at any alignment, so no alignment
@@ -265,6 +268,9 @@ CopyCache& copy_cache() {
 constexpr size_t kCopyCacheCapacity = 64;
 
 // Finds or builds the tables for (out, in, sizes) with elements of unit bytes.
+// The caller holds the cache mutex and keeps it until its launch is enqueued:
+// an eviction by another thread synchronises the device before it frees a
+// table, which is only safe once every user of that table has been queued.
 int cached_tables(void* const* out, const void* const* in, const size_t* sizes, int n,
                   uint32_t unit, DevTables* result) {
   std::vector<uint64_t> key;
@@ -277,7 +283,6 @@ int cached_tables(void* const* out, const void* const* in, const size_t* sizes, 
     key.push_back((uint64_t)sizes[i]);
   }
   CopyCache& c = copy_cache();
-  std::lock_guard<std::mutex> g(c.mu);
   for (auto it = c.lru.begin(); it != c.lru.end(); ++it) {
     if (it->key == key) {
       c.lru.splice(c.lru.begin(), c.lru, it);
@@ -336,6 +341,7 @@ int hvdhip_batched_d2d_memcpy(void* const* out, const void* const* in, const siz
   if (rc) return rc;
   if (num_copies == 0) return ok();
   DevTables t;
+  std::lock_guard<std::mutex> g(copy_cache().mu);
   rc = cached_tables(out, in, sizes, num_copies, 1, &t);
   if (rc) return rc;
   rc = launch_xfer<Copy<uint8_t>, kDirect>(t, 0, {}, static_cast<hipStream_t>(stream));
@@ -358,6 +364,7 @@ int hvdhip_batched_scaled_d2d_memcpy(void* const* out, const void* const* in,
       return fail(HVDHIP_ERR_INVALID_ARGUMENT, "copy %d is not aligned to its element size", i);
   }
   DevTables t;
+  std::lock_guard<std::mutex> g(copy_cache().mu);
   rc = cached_tables(out, in, sizes, num_copies, es, &t);
   if (rc) return rc;
   rc = launch_same_dtype<kDirect>(t, 0, scale_factor, dtype, static_cast<hipStream_t>(stream));

@@ -233,6 +233,47 @@ def test_batched_scaled_d2d_memcpy(gpu, orc, dtype, scale):
         assert np.array_equal(out[o:o + c * es], want.view(np.uint8))
 
 
+def test_batched_copy_cache_eviction_from_several_threads(gpu):
+    # more distinct copy sets than the table cache holds (64), issued from four threads on four streams
+    import threading
+    import horovod_amd
+    rng = np.random.default_rng(12)
+    nsets, per = 40, 6
+    src = Arena(4 << 20)
+    dst = Arena(4 << 20, fill=0x5A)
+    sets = []
+    for s_ in range(4 * nsets):
+        sizes = [int(x) for x in rng.integers(1, 3000, per)]
+        so = [src.alloc(n, align=16) for n in sizes]
+        do = [dst.alloc(n, align=16) for n in sizes]
+        for o, n in zip(so, sizes):
+            src.host[o:o + n] = rng.integers(0, 256, n, dtype=np.uint8)
+        sets.append((so, do, sizes))
+    src.upload(), dst.upload()
+    errors = []
+
+    def worker(t):
+        try:
+            horovod_amd.lib().hvdhip_set_device(0)
+            st = horovod_amd.Stream()
+            for rep in range(2):
+                for so, do, sizes in sets[t * nsets:(t + 1) * nsets]:
+                    gpu.H.batched_d2d_memcpy([dst.ptr(o) for o in do], [src.ptr(o) for o in so], sizes, st)
+            st.synchronize()
+            st.destroy()
+        except Exception as e:  # pragma: no cover
+            errors.append(e)
+
+    ts = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    [t.start() for t in ts]
+    [t.join() for t in ts]
+    assert not errors, errors
+    out = dst.download()
+    for so, do, sizes in sets:
+        for s_, d_, n in zip(so, do, sizes):
+            assert np.array_equal(out[d_:d_ + n], src.host[s_:s_ + n])
+
+
 def test_rejected_arguments(gpu):
     import horovod_amd
     L = horovod_amd.lib()
