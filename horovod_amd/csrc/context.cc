@@ -95,17 +95,16 @@ int upload_chunks(const std::vector<Chunk>& chunks, DevTables* out) {
   return 0;
 }
 
-int build_tables(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t tensor_es,
-                 uint32_t buffer_es, DevTables* out) {
-  if (chunk_units == 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "chunk_units is zero");
+uint64_t count_chunks(const std::vector<Seg>& segs, uint32_t chunk_units) {
   uint64_t nchunks = 0;
   for (const Seg& s : segs) nchunks += (s.n + chunk_units - 1) / chunk_units;
-  if (nchunks > 0x7fffffffull)
-    return fail(HVDHIP_ERR_TOO_LARGE, "plan needs %llu workgroups; the limit is 2^31-1",
-                (unsigned long long)nchunks);
-  std::vector<Chunk> chunks;
-  chunks.reserve((size_t)nchunks);
+  return nchunks > 0x7fffffffull ? ~0ull : nchunks;
+}
+
+void fill_chunks(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t tensor_es,
+                 uint32_t buffer_es, Chunk* out) {
   for (const Seg& s : segs) {
+    const uint64_t nbytes = s.n * buffer_es;
     for (uint64_t start = 0; start < s.n; start += chunk_units) {
       const uint64_t left = s.n - start;
       Chunk c;
@@ -113,11 +112,19 @@ int build_tables(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t te
       c.output = s.output + start * tensor_es;
       c.off = s.off + start * buffer_es;
       c.n = (uint32_t)(left < chunk_units ? left : chunk_units);
-      const uint64_t nbytes = s.n * buffer_es;
       c.pad = left <= chunk_units ? (uint32_t)((16 - (nbytes & 15)) & 15) : 0;
-      chunks.push_back(c);
+      *out++ = c;
     }
   }
+}
+
+int build_tables(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t tensor_es,
+                 uint32_t buffer_es, DevTables* out) {
+  if (chunk_units == 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "chunk_units is zero");
+  const uint64_t nchunks = count_chunks(segs, chunk_units);
+  if (nchunks == ~0ull) return fail(HVDHIP_ERR_TOO_LARGE, "plan needs more than 2^31-1 workgroups");
+  std::vector<Chunk> chunks((size_t)nchunks);
+  fill_chunks(segs, chunk_units, tensor_es, buffer_es, chunks.data());
   return upload_chunks(chunks, out);
 }
 

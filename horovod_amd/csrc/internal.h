@@ -101,6 +101,12 @@ struct DevTables {
 // segments get no chunk.
 int build_tables(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t tensor_es,
                  uint32_t buffer_es, DevTables* out);
+// The two halves of build_tables for callers that stage the table themselves:
+// the number of chunks the segments need (0xffffffffffffffff if over the
+// limit), and the fill of a caller-provided array of that many entries.
+uint64_t count_chunks(const std::vector<Seg>& segs, uint32_t chunk_units);
+void fill_chunks(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t tensor_es,
+                 uint32_t buffer_es, Chunk* out);
 // Uploads a ready-made chunk table.
 int upload_chunks(const std::vector<Chunk>& chunks, DevTables* out);
 int free_tables(DevTables* t);

@@ -251,28 +251,99 @@ int launch_contig(const void* in, void* out, int64_t n, typename Op::P p, hipStr
 }
 
 // ---- cache of tables for the array-taking entry points ----------------
+//
+// The reference passes its copy descriptors by value with every launch, so a
+// caller of these entry points expects no set-up cost.  A hit costs a key
+// comparison.  A miss allocates nothing and never waits for the device in the
+// steady state: the table is written straight into a pinned staging buffer
+// that belongs to the cache entry, copied to the entry's device buffer with an
+// asynchronous copy on the caller's stream, and the kernel follows on the
+// same stream.  Evicted entries hand their buffers to the next miss; before
+// that, the entry's last-use event is waited for (normally long complete).
+
+struct TableBuf {
+  void* dev = nullptr;
+  void* pinned = nullptr;
+  size_t cap = 0;
+};
 
 struct CachedCopy {
   std::vector<uint64_t> key;  // unit size, n, then out/in/size triples
-  DevTables tables;
+  DevTables tables;           // tables.alloc is not owned: it aliases buf.dev
+  TableBuf buf;
+  hipEvent_t done = nullptr;        // recorded after every launch that reads the table
+  hipStream_t last_stream = nullptr;
+  bool several_streams = false;     // used on more than one stream since it was built
 };
 
 struct CopyCache {
   std::mutex mu;
   std::list<CachedCopy> lru;  // front = most recent
+  std::vector<TableBuf> spare;
 };
 CopyCache& copy_cache() {
   static CopyCache* c = new CopyCache();
   return *c;
 }
 constexpr size_t kCopyCacheCapacity = 64;
+constexpr size_t kSpareBufs = 8;
 
-// Finds or builds the tables for (out, in, sizes) with elements of unit bytes.
-// The caller holds the cache mutex and keeps it until its launch is enqueued:
-// an eviction by another thread synchronises the device before it frees a
-// table, which is only safe once every user of that table has been queued.
+void release_buf(TableBuf* b) {
+  if (b->dev) (void)hipFree(b->dev);
+  if (b->pinned) (void)hipHostFree(b->pinned);
+  *b = TableBuf();
+}
+
+// A device + pinned buffer pair of at least `bytes`: the smallest spare that fits, else new.
+int acquire_buf(CopyCache& c, size_t bytes, TableBuf* out) {
+  size_t best = c.spare.size();
+  for (size_t i = 0; i < c.spare.size(); ++i)
+    if (c.spare[i].cap >= bytes && (best == c.spare.size() || c.spare[i].cap < c.spare[best].cap)) best = i;
+  if (best != c.spare.size()) {
+    *out = c.spare[best];
+    c.spare.erase(c.spare.begin() + (long)best);
+    return 0;
+  }
+  size_t cap = 4096;
+  while (cap < bytes) cap *= 2;
+  TableBuf b;
+  hipError_t e = hipMalloc(&b.dev, cap);
+  if (e == hipSuccess) e = hipHostMalloc(&b.pinned, cap, hipHostMallocDefault);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    release_buf(&b);
+    return fail(e == hipErrorOutOfMemory ? HVDHIP_ERR_OUT_OF_MEMORY : (int)e,
+                "allocating %zu bytes for a copy table failed: %s", cap, hipGetErrorString(e));
+  }
+  b.cap = cap;
+  *out = b;
+  return 0;
+}
+
+// Takes the least recently used entry out of the cache once nothing on the device can
+// still read its table, and keeps its buffers for reuse.
+int evict_one(CopyCache& c) {
+  CachedCopy& victim = c.lru.back();
+  if (victim.several_streams) {
+    HVDHIP_CHECK(hipDeviceSynchronize());
+  } else if (victim.done) {
+    HVDHIP_CHECK(hipEventSynchronize(victim.done));
+  }
+  if (victim.done) (void)hipEventDestroy(victim.done);
+  if (c.spare.size() < kSpareBufs) {
+    c.spare.push_back(victim.buf);
+  } else {
+    release_buf(&victim.buf);
+  }
+  c.lru.pop_back();
+  return 0;
+}
+
+// Finds or builds the table for (out, in, sizes) with elements of unit bytes; a newly
+// built table is uploaded asynchronously on `stream`.  The caller holds the cache mutex,
+// launches on `stream`, then calls mark_used() before releasing the mutex.
 int cached_tables(void* const* out, const void* const* in, const size_t* sizes, int n,
-                  uint32_t unit, DevTables* result) {
+                  uint32_t unit, hipStream_t stream, CachedCopy** result) {
   std::vector<uint64_t> key;
   key.reserve(2 + 3 * (size_t)n);
   key.push_back(unit);
@@ -286,25 +357,56 @@ int cached_tables(void* const* out, const void* const* in, const size_t* sizes, 
   for (auto it = c.lru.begin(); it != c.lru.end(); ++it) {
     if (it->key == key) {
       c.lru.splice(c.lru.begin(), c.lru, it);
-      *result = c.lru.front().tables;
+      CachedCopy* hit = &c.lru.front();
+      // The table was uploaded asynchronously on the stream that built it; another stream
+      // must not read it earlier.  `done` was recorded on that stream after the upload.
+      if (stream != hit->last_stream) HVDHIP_CHECK(hipStreamWaitEvent(stream, hit->done, 0));
+      *result = hit;
       return 0;
     }
   }
   std::vector<Seg> segs((size_t)n);
   for (int i = 0; i < n; ++i)
-    segs[i] = Seg{(uint64_t)(uintptr_t)in[i], (uint64_t)(uintptr_t)out[i], 0, sizes[i] / unit};
-  CachedCopy entry;
-  entry.key.swap(key);
-  int rc = build_tables(segs, chunk_bytes(Family::kXfer) / unit, unit, unit, &entry.tables);
-  if (rc) return rc;
+    segs[(size_t)i] = Seg{(uint64_t)(uintptr_t)in[i], (uint64_t)(uintptr_t)out[i], 0, sizes[i] / unit};
+  const uint32_t chunk_units = chunk_bytes(Family::kXfer) / unit;
+  const uint64_t nchunks = count_chunks(segs, chunk_units);
+  if (nchunks == ~0ull) return fail(HVDHIP_ERR_TOO_LARGE, "the copies need more than 2^31-1 workgroups");
   if (c.lru.size() >= kCopyCacheCapacity) {
-    // Tables may still be read by queued kernels: wait before freeing.
-    HVDHIP_CHECK(hipDeviceSynchronize());
-    free_tables(&c.lru.back().tables);
-    c.lru.pop_back();
+    int rc = evict_one(c);
+    if (rc) return rc;
   }
+  CachedCopy entry;
+  const size_t bytes = (size_t)nchunks * sizeof(Chunk);
+  int rc = acquire_buf(c, bytes ? bytes : 32, &entry.buf);
+  if (rc) return rc;
+  hipError_t e = hipEventCreateWithFlags(&entry.done, hipEventDisableTiming);
+  if (e == hipSuccess && nchunks) {
+    fill_chunks(segs, chunk_units, unit, unit, static_cast<Chunk*>(entry.buf.pinned));
+    e = hipMemcpyAsync(entry.buf.dev, entry.buf.pinned, bytes, hipMemcpyHostToDevice, stream);
+  }
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    if (entry.done) (void)hipEventDestroy(entry.done);
+    // the copy may have been queued: do not hand the buffers on before the stream is idle
+    (void)hipStreamSynchronize(stream);
+    c.spare.push_back(entry.buf);
+    return fail((int)e, "staging a copy table failed: %s", hipGetErrorString(e));
+  }
+  entry.key.swap(key);
+  entry.tables.alloc = nullptr;
+  entry.tables.chunks = static_cast<Chunk*>(entry.buf.dev);
+  entry.tables.nchunks = (uint32_t)nchunks;
+  entry.last_stream = stream;
   c.lru.push_front(std::move(entry));
-  *result = c.lru.front().tables;
+  *result = &c.lru.front();
+  return 0;
+}
+
+// Records that `stream` now holds work reading the entry's table.
+int mark_used(CachedCopy* entry, hipStream_t stream) {
+  if (stream != entry->last_stream) entry->several_streams = true;
+  entry->last_stream = stream;
+  HVDHIP_CHECK(hipEventRecord(entry->done, stream));
   return 0;
 }
 
@@ -340,11 +442,14 @@ int hvdhip_batched_d2d_memcpy(void* const* out, const void* const* in, const siz
   int rc = check_arrays(out, in, sizes, num_copies);
   if (rc) return rc;
   if (num_copies == 0) return ok();
-  DevTables t;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  CachedCopy* entry = nullptr;
   std::lock_guard<std::mutex> g(copy_cache().mu);
-  rc = cached_tables(out, in, sizes, num_copies, 1, &t);
+  rc = cached_tables(out, in, sizes, num_copies, 1, s, &entry);
   if (rc) return rc;
-  rc = launch_xfer<Copy<uint8_t>, kDirect>(t, 0, {}, static_cast<hipStream_t>(stream));
+  rc = launch_xfer<Copy<uint8_t>, kDirect>(entry->tables, 0, {}, s);
+  int rc2 = mark_used(entry, s);
+  if (rc == 0) rc = rc2;
   return rc ? rc : ok();
 }
 
@@ -363,11 +468,14 @@ int hvdhip_batched_scaled_d2d_memcpy(void* const* out, const void* const* in,
     if (((uintptr_t)out[i] | (uintptr_t)in[i]) % es)
       return fail(HVDHIP_ERR_INVALID_ARGUMENT, "copy %d is not aligned to its element size", i);
   }
-  DevTables t;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  CachedCopy* entry = nullptr;
   std::lock_guard<std::mutex> g(copy_cache().mu);
-  rc = cached_tables(out, in, sizes, num_copies, es, &t);
+  rc = cached_tables(out, in, sizes, num_copies, es, s, &entry);
   if (rc) return rc;
-  rc = launch_same_dtype<kDirect>(t, 0, scale_factor, dtype, static_cast<hipStream_t>(stream));
+  rc = launch_same_dtype<kDirect>(entry->tables, 0, scale_factor, dtype, s);
+  int rc2 = mark_used(entry, s);
+  if (rc == 0) rc = rc2;
   return rc ? rc : ok();
 }
 

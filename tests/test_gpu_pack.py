@@ -274,6 +274,33 @@ def test_batched_copy_cache_eviction_from_several_threads(gpu):
             assert np.array_equal(out[d_:d_ + n], src.host[s_:s_ + n])
 
 
+def test_batched_copy_table_built_on_one_stream_used_on_another(gpu):
+    # a miss uploads its table asynchronously on the calling stream; a hit from another stream
+    # right behind it must wait for that upload
+    import horovod_amd
+    rng = np.random.default_rng(13)
+    a, b = horovod_amd.Stream(), horovod_amd.Stream()
+    n = 3000
+    sizes = [int(x) for x in rng.integers(1, 9000, n)]
+    src = Arena(sum(sizes) + 32 * n + 4096)
+    so = [src.alloc(x, align=16) for x in sizes]
+    for o, x in zip(so, sizes):
+        src.host[o:o + x] = rng.integers(0, 256, x, dtype=np.uint8)
+    src.upload()
+    for rep in range(5):
+        dst = Arena(src.capacity + 64 * rep, fill=0x5A)
+        do = [dst.alloc(x, misalign=rep, align=16) for x in sizes]
+        dst.upload()
+        out_ptrs, in_ptrs = [dst.ptr(o) for o in do], [src.ptr(o) for o in so]
+        gpu.H.batched_d2d_memcpy(out_ptrs, in_ptrs, sizes, a)   # miss: builds and uploads on a
+        gpu.H.batched_d2d_memcpy(out_ptrs, in_ptrs, sizes, b)   # hit on b
+        a.synchronize(), b.synchronize()
+        out = dst.download()
+        for s_, d_, x in zip(so, do, sizes):
+            assert np.array_equal(out[d_:d_ + x], src.host[s_:s_ + x])
+    a.destroy(), b.destroy()
+
+
 def test_rejected_arguments(gpu):
     import horovod_amd
     L = horovod_amd.lib()
