@@ -181,7 +181,18 @@ hvdhip_fusion_plan* GPUAllreduce::PlanFor(const std::vector<TensorTableEntry>& e
     key.push_back((uint64_t)e.num_elements);
   }
   auto it = plans_.find(key);
-  if (it != plans_.end()) return it->second;
+  if (it != plans_.end()) {
+    plan_order_.remove(key);
+    plan_order_.push_front(key);
+    return it->second;
+  }
+  if (plans_.size() >= kMaxPlans) {
+    // destroying a plan waits for the device, so no queued kernel can still read its tables
+    auto victim = plans_.find(plan_order_.back());
+    hvdhip_fusion_plan_destroy(victim->second);
+    plans_.erase(victim);
+    plan_order_.pop_back();
+  }
   std::vector<const void*> tensors;
   std::vector<void*> outputs;
   std::vector<int64_t> counts;
@@ -195,6 +206,7 @@ hvdhip_fusion_plan* GPUAllreduce::PlanFor(const std::vector<TensorTableEntry>& e
                            hvdhip_fusion_plan_create(tensors.data(), outputs.data(), counts.data(), (int)entries.size(),
                                                      (int)entries[0].dtype, (int)entries[0].dtype, &plan));
   plans_[key] = plan;
+  plan_order_.push_front(key);
   return plan;
 }
 

@@ -22,6 +22,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <functional>
+#include <list>
 #include <map>
 #include <memory>
 #include <queue>
@@ -167,7 +168,11 @@ private:
   GPUContext* gpu_context_;
   GlobalState* global_state_;
   GPUOpContext gpu_op_context_;
+  // At most kMaxPlans resident plans, least recently used first out, so that a framework
+  // that hands over fresh tensor addresses every step cannot grow the cache without bound.
+  static constexpr size_t kMaxPlans = 128;
   std::map<std::vector<uint64_t>, hvdhip_fusion_plan*> plans_;
+  std::list<std::vector<uint64_t>> plan_order_;  // front = most recently used
 };
 
 // The fusion-buffer hooks of the allgather op (ops/collective_operations.cc:200-275,

@@ -154,6 +154,26 @@ def test_async_completion_and_elastic_polling_paths(gpu, orc, adapter):
             h.close()
 
 
+def test_plan_cache_is_bounded_when_tensor_addresses_keep_changing(gpu, orc, adapter):
+    # 140 distinct entry lists through one op: the cache holds at most 128 plans and results stay right
+    rng = np.random.default_rng(8)
+    v = rng.standard_normal(64 * 142).astype(np.float32)
+    d_v, d_o = gpu.upload(v), gpu.empty(v.nbytes, fill=0)
+    h = Harness(adapter, gpu, num_streams=1)
+    try:
+        for i in range(140):
+            t = [d_v.data_ptr() + 256 * i, d_v.data_ptr() + 256 * (i + 1)]
+            o = [d_o.data_ptr() + 256 * i, d_o.data_ptr() + 256 * (i + 1)]
+            rc, msg = h.allreduce(t, o, [64, 64], F32, 0.5, 1.0)
+            assert rc == 0, msg
+        _, plans = h.state()
+        assert plans == 128
+        got = gpu.download(d_o, np.float32)
+        assert np.array_equal(got[:64 * 141], orc.scale_buffer(v[:64 * 141], 0.5, F32))
+    finally:
+        h.close()
+
+
 def test_timeline_hooks_record_an_event_after_every_stage(gpu, orc, adapter):
     # ops/nccl_operations.cc:173-175,195-197,203-205 and ops/gpu_operations.cc:45-47
     rng = np.random.default_rng(6)
