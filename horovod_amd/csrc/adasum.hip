@@ -357,7 +357,7 @@ int hvdhip_adasum_plan_create(const int* tensor_counts, int nlayers, int dtype,
       chunks.push_back(Chunk{off + start, (uint64_t)i, 0, (uint32_t)(left < chunk_units ? left : chunk_units), 0});
     }
     layers[(size_t)i].count = (uint32_t)chunks.size() - layers[(size_t)i].first;
-    if (chunks.size() > 0x7fffffffull) return fail(HVDHIP_ERR_TOO_LARGE, "too many chunks");
+    if (chunks.size() > kMaxWorkgroups) return fail(HVDHIP_ERR_TOO_LARGE, "the vectors need more than 2^23 workgroups");
     off += n;
   }
   hvdhip_adasum_plan* p = new hvdhip_adasum_plan();

@@ -71,8 +71,9 @@ uint32_t chunk_bytes(Family f) {
 }
 
 int upload_chunks(const std::vector<Chunk>& chunks, DevTables* out) {
-  if (chunks.size() > 0x7fffffffull)
-    return fail(HVDHIP_ERR_TOO_LARGE, "plan needs %zu workgroups; the limit is 2^31-1", chunks.size());
+  if (chunks.size() > kMaxWorkgroups)
+    return fail(HVDHIP_ERR_TOO_LARGE, "plan needs %zu workgroups; the limit is %llu", chunks.size(),
+                (unsigned long long)kMaxWorkgroups);
   const size_t total = chunks.empty() ? 256 : chunks.size() * sizeof(Chunk);
   void* dev = nullptr;
   hipError_t e = hipMalloc(&dev, total);
@@ -98,7 +99,7 @@ int upload_chunks(const std::vector<Chunk>& chunks, DevTables* out) {
 uint64_t count_chunks(const std::vector<Seg>& segs, uint32_t chunk_units) {
   uint64_t nchunks = 0;
   for (const Seg& s : segs) nchunks += (s.n + chunk_units - 1) / chunk_units;
-  return nchunks > 0x7fffffffull ? ~0ull : nchunks;
+  return nchunks > kMaxWorkgroups ? ~0ull : nchunks;
 }
 
 void fill_chunks(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t tensor_es,
@@ -122,7 +123,7 @@ int build_tables(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t te
                  uint32_t buffer_es, DevTables* out) {
   if (chunk_units == 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "chunk_units is zero");
   const uint64_t nchunks = count_chunks(segs, chunk_units);
-  if (nchunks == ~0ull) return fail(HVDHIP_ERR_TOO_LARGE, "plan needs more than 2^31-1 workgroups");
+  if (nchunks == ~0ull) return fail(HVDHIP_ERR_TOO_LARGE, "plan needs more than 2^23 workgroups");
   std::vector<Chunk> chunks((size_t)nchunks);
   fill_chunks(segs, chunk_units, tensor_es, buffer_es, chunks.data());
   return upload_chunks(chunks, out);

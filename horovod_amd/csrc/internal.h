@@ -52,6 +52,10 @@ inline int64_t dtype_size(int dtype) {
 // Threads per workgroup of every streaming kernel: four wave64 wavefronts.
 constexpr int kWG = 256;
 
+// A launch may not exceed 2^32 - 1 threads in x.  Contiguous kernels cover larger buffers
+// in slices of kMaxWorkgroups workgroups; a plan that needs more is refused.
+constexpr uint64_t kMaxWorkgroups = 1ull << 23;
+
 // Bytes of the wider side that one workgroup moves.  Measured on MI355X with
 // buffers far larger than the 256 MB Infinity Cache: one 16-byte access per
 // lane and workgroup (4 KiB) with non-temporal hints streams at about 80 % of

@@ -92,15 +92,19 @@ __global__ __launch_bounds__(kWG) void reduce_k(T* resident, Peers<K> peers, uin
 
 template <typename T, int K>
 int launch_k(void* resident, const void* const* incoming, int64_t n, hipStream_t stream) {
-  // Fewer bytes per workgroup as more peers stream in, to keep loads in flight similar.
-  uint32_t tile = chunk_bytes(Family::kReduce) / (uint32_t)sizeof(T);
-  const uint64_t blocks = ((uint64_t)n + tile - 1) / tile;
-  if (blocks > 0x7fffffffull) return fail(HVDHIP_ERR_TOO_LARGE, "chunk of %lld elements is too large", (long long)n);
-  Peers<K> peers;
-  for (int k = 0; k < K; ++k) peers.p[k] = incoming[k];
-  hipLaunchKernelGGL((reduce_k<T, K>), dim3((uint32_t)blocks), dim3(kWG), 0, stream,
-                     static_cast<T*>(resident), peers, (uint64_t)n, tile);
-  HVDHIP_CHECK_LAUNCH("reduce_k");
+  const uint32_t tile = chunk_bytes(Family::kReduce) / (uint32_t)sizeof(T);
+  uint64_t done = 0, left = (uint64_t)n;
+  while (left > 0) {  // one launch unless the chunk needs more than kMaxWorkgroups workgroups
+    const uint64_t slice = left < kMaxWorkgroups * tile ? left : kMaxWorkgroups * tile;
+    const uint32_t blocks = (uint32_t)((slice + tile - 1) / tile);
+    Peers<K> peers;
+    for (int k = 0; k < K; ++k) peers.p[k] = static_cast<const T*>(incoming[k]) + done;
+    hipLaunchKernelGGL((reduce_k<T, K>), dim3(blocks), dim3(kWG), 0, stream, static_cast<T*>(resident) + done,
+                       peers, slice, tile);
+    HVDHIP_CHECK_LAUNCH("reduce_k");
+    done += slice;
+    left -= slice;
+  }
   return 0;
 }
 

@@ -240,13 +240,21 @@ bool scalable(int dtype) {
 
 template <class Op>
 int launch_contig(const void* in, void* out, int64_t n, typename Op::P p, hipStream_t stream) {
-  const uint32_t tile = chunk_bytes(Family::kXfer) / (uint32_t)std::max(sizeof(typename Op::S), sizeof(typename Op::D));
-  const uint64_t blocks = ((uint64_t)n + tile - 1) / tile;
-  if (blocks > 0x7fffffffull) return fail(HVDHIP_ERR_TOO_LARGE, "buffer of %lld elements is too large", (long long)n);
-  hipLaunchKernelGGL((contig_k<Op>), dim3((uint32_t)blocks), dim3(kWG), 0, stream,
-                     static_cast<const typename Op::S*>(in), static_cast<typename Op::D*>(out),
-                     (uint64_t)n, tile, p);
-  HVDHIP_CHECK_LAUNCH("contig_k");
+  typedef typename Op::S S;
+  typedef typename Op::D D;
+  const uint32_t tile = chunk_bytes(Family::kXfer) / (uint32_t)std::max(sizeof(S), sizeof(D));
+  const S* src = static_cast<const S*>(in);
+  D* dst = static_cast<D*>(out);
+  uint64_t left = (uint64_t)n;
+  while (left > 0) {  // one launch unless the buffer needs more than kMaxWorkgroups workgroups
+    const uint64_t slice = std::min<uint64_t>(left, kMaxWorkgroups * tile);
+    const uint32_t blocks = (uint32_t)((slice + tile - 1) / tile);
+    hipLaunchKernelGGL((contig_k<Op>), dim3(blocks), dim3(kWG), 0, stream, src, dst, slice, tile, p);
+    HVDHIP_CHECK_LAUNCH("contig_k");
+    src += slice;
+    dst += slice;
+    left -= slice;
+  }
   return 0;
 }
 
@@ -370,7 +378,7 @@ int cached_tables(void* const* out, const void* const* in, const size_t* sizes, 
     segs[(size_t)i] = Seg{(uint64_t)(uintptr_t)in[i], (uint64_t)(uintptr_t)out[i], 0, sizes[i] / unit};
   const uint32_t chunk_units = chunk_bytes(Family::kXfer) / unit;
   const uint64_t nchunks = count_chunks(segs, chunk_units);
-  if (nchunks == ~0ull) return fail(HVDHIP_ERR_TOO_LARGE, "the copies need more than 2^31-1 workgroups");
+  if (nchunks == ~0ull) return fail(HVDHIP_ERR_TOO_LARGE, "the copies need more than 2^23 workgroups");
   if (c.lru.size() >= kCopyCacheCapacity) {
     int rc = evict_one(c);
     if (rc) return rc;

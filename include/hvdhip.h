@@ -52,6 +52,8 @@ enum hvdhip_dtype {
  * (ops/collective_operations.cc:141-144, ops/cuda/cuda_kernels.cu:182-185,317-319). */
 #define HVDHIP_ERR_UNSUPPORTED_DTYPE (-2)
 #define HVDHIP_ERR_OUT_OF_MEMORY (-3)
+/* A plan or batched copy needs more than 2^23 workgroups (32 GiB at 4 KiB each) in one launch.
+ * Contiguous entry points (scale, reduce) have no such limit: they slice. */
 #define HVDHIP_ERR_TOO_LARGE (-4)
 
 /* Flags of hvdhip_fusion_pack(). */

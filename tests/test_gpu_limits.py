@@ -66,6 +66,26 @@ def test_reduce_and_adasum_beyond_2_31_elements(gpu, orc):
     plan.destroy()
 
 
+def test_contiguous_kernels_slice_beyond_one_launch(gpu):
+    # 33 GiB of int8: more than 2^23 workgroups of 4 KiB, so scale and reduce run as two launches each
+    n = (33 << 30) + 777
+    x = torch.full((n,), 4, dtype=torch.int8, device="cuda")
+    y = torch.full((n,), 7, dtype=torch.int8, device="cuda")
+    x[-1] = 8
+    torch.cuda.synchronize()
+    gpu.H.scale_buffer(x.data_ptr(), x.data_ptr(), n, 2.5, I8, gpu.stream)
+    gpu.sync()
+    assert int(x[:-1].min()) == 10 and int(x[:-1].max()) == 10 and int(x[-1]) == 20
+    gpu.H.reduce_sum(x.data_ptr(), y.data_ptr(), n, I8, gpu.stream)
+    gpu.sync()
+    assert int(x[:-1].min()) == 17 and int(x[:-1].max()) == 17 and int(x[-1]) == 27
+    # a plan of that size is refused rather than mis-launched
+    import horovod_amd
+    with pytest.raises(horovod_amd.HvdHipError) as e:
+        gpu.H.FusionPlan([x.data_ptr()], [y.data_ptr()], [n], U8)
+    assert e.value.code == -4
+
+
 def test_pipeline_replays_from_a_hip_graph(gpu, orc):
     """pack -> reduce -> unpack captured once and replayed: the entry points only launch kernels
     (no allocation, no memset), so they can be captured; every replay must equal the eager result."""
