@@ -347,6 +347,7 @@ def extras(steps, warmup):
         out[name] = {"GB/s": round(ab / sec / 1e9, 1), "frac_of_hbm_peak": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4),
                      "ms": round(sec * 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1), "cycles": len(pipe.cycles),
                      "streams": streams, "peers": peers, "reduce": "k-way" if kway else "per-peer",
+                     "completion_event_per_cycle": pipe.completion_events,
                      "replicas_rotated": replicas}
         for _, _, pipe, _ in reps:
             pipe.destroy()

@@ -14,10 +14,12 @@ current_nccl_stream after every op (ops/gpu_operations.cc:101-103).
 
 This module only sequences calls; all arithmetic happens in libhvdhip.so.
 """
+import ctypes
+
 import torch
 
 from . import host as H
-from ._lib import DTYPE, dtype_size
+from ._lib import DTYPE, check, dtype_size, lib
 from .workloads import FUSION_THRESHOLD, fuse
 
 
@@ -41,7 +43,11 @@ class AllreducePipeline:
     share)."""
 
     def __init__(self, tensor_ptrs, output_ptrs, counts, tensor_dtype, buffer_dtype=None,
-                 threshold=FUSION_THRESHOLD, num_streams=1):
+                 threshold=FUSION_THRESHOLD, num_streams=1, completion_events=None):
+        """completion_events: record a pooled event after every cycle and wait on those in
+        synchronize(), as GPUOpContext::FinalizeGPUQueue does (about 2 us of stream time per
+        event).  Default: on when cycles alternate over several streams, off for one stream,
+        where synchronize() simply waits for the stream."""
         self.tensor_dtype = int(tensor_dtype)
         self.buffer_dtype = int(tensor_dtype if buffer_dtype is None else buffer_dtype)
         ts, bs = dtype_size(self.tensor_dtype), dtype_size(self.buffer_dtype)
@@ -64,6 +70,8 @@ class AllreducePipeline:
             cyc.payload_in, cyc.payload_buf, cyc.payload_out = n * ts, n * bs, n * ts
             self.cycles.append(cyc)
         self.streams = [H.Stream() for _ in range(num_streams)]
+        self.completion_events = (num_streams > 1) if completion_events is None else bool(completion_events)
+        self.pending = []  # (stream, event) recorded after each cycle
         self.buffers = [torch.empty(max(max_len, 16), dtype=torch.uint8, device="cuda") for _ in range(num_streams)]
         torch.cuda.synchronize()
 
@@ -100,8 +108,20 @@ class AllreducePipeline:
             elif postscale != 1.0:
                 t, o, n = cyc.single
                 H.scale_buffer(o, o, n, postscale, self.tensor_dtype, s)
+            # completion marker from the event pool (ops/gpu_operations.cc:50-56); the finalizer waits on it
+            if self.completion_events:
+                ev = ctypes.c_void_p()
+                check(lib().hvdhip_event_acquire(s.handle, ctypes.byref(ev)), "hvdhip_event_acquire")
+                check(lib().hvdhip_event_record(ev, s.handle), "hvdhip_event_record")
+                self.pending.append((s, ev))
 
     def synchronize(self):
+        """Waits for every cycle's completion event and returns the events to their pools
+        (GPUContext::WaitForEvents, ops/cuda_operations.cc:102-148)."""
+        for s, ev in self.pending:
+            check(lib().hvdhip_event_synchronize(ev), "hvdhip_event_synchronize")
+            check(lib().hvdhip_event_release(s.handle, ev), "hvdhip_event_release")
+        self.pending = []
         for s in self.streams:
             s.synchronize()
 
@@ -119,6 +139,7 @@ class AllreducePipeline:
         return total
 
     def destroy(self):
+        self.synchronize()
         for cyc in self.cycles:
             if cyc.plan is not None:
                 cyc.plan.destroy()

@@ -63,7 +63,8 @@ def test_c1_resnet50_fp32_pack_prescale_sum_unpack(gpu, orc):
     offs, img, vals = _host_set(counts, 4, lambda n: (rng.standard_normal(n) * 1e-3).astype(np.float32))
     d_in = torch.from_numpy(img).cuda()
     d_out = torch.zeros_like(d_in)
-    pipe = AllreducePipeline([d_in.data_ptr() + o for o in offs], [d_out.data_ptr() + o for o in offs], counts, F32)
+    pipe = AllreducePipeline([d_in.data_ptr() + o for o in offs], [d_out.data_ptr() + o for o in offs], counts, F32,
+                             completion_events=True)
     assert len(pipe.cycles) == 2  # 102.2 MB through a 64 MiB threshold
     peers, peer_vals = _peer_images(pipe, counts, 4, lambda n: (prng.standard_normal(n) * 1e-3).astype(np.float32))
     pipe.run(0.125, 1.0, lambda ci, p: peers[ci].data_ptr(), 1)
