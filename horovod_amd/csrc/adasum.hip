@@ -229,6 +229,7 @@ using namespace hvdhip;
 struct hvdhip_adasum_plan {
   int nlayers = 0;
   int dtype = 0;
+  int device = 0;  // the device that holds the tables and results
   int64_t total = 0;
   DevTables tables;
   Layer* layers = nullptr;    // device, nlayers entries
@@ -314,8 +315,10 @@ constexpr size_t kOneLayerCapacity = 256;
 // blocking entry point, finished): eviction destroys plans, and plans carry state.
 int one_layer_plan(int count, int dtype, hvdhip_adasum_plan** out) {
   OneLayerCache& c = one_layer_cache();
+  int device = 0;
+  HVDHIP_CHECK(hipGetDevice(&device));
   for (auto it = c.lru.begin(); it != c.lru.end(); ++it) {
-    if ((*it)->total == count && (*it)->dtype == dtype) {
+    if ((*it)->total == count && (*it)->dtype == dtype && (*it)->device == device) {
       c.lru.splice(c.lru.begin(), c.lru, it);
       *out = c.lru.front();
       return 0;
@@ -364,6 +367,7 @@ int hvdhip_adasum_plan_create(const int* tensor_counts, int nlayers, int dtype,
   p->nlayers = nlayers;
   p->dtype = dtype;
   p->total = (int64_t)off;
+  (void)hipGetDevice(&p->device);
   int rc = upload_chunks(chunks, &p->tables);
   if (rc) {
     delete p;

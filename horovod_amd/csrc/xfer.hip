@@ -276,7 +276,7 @@ struct TableBuf {
 };
 
 struct CachedCopy {
-  std::vector<uint64_t> key;  // unit size, n, then out/in/size triples
+  std::vector<uint64_t> key;  // device and unit size, n, then out/in/size triples
   DevTables tables;           // tables.alloc is not owned: it aliases buf.dev
   TableBuf buf;
   hipEvent_t done = nullptr;        // recorded after every launch that reads the table
@@ -352,9 +352,11 @@ int evict_one(CopyCache& c) {
 // launches on `stream`, then calls mark_used() before releasing the mutex.
 int cached_tables(void* const* out, const void* const* in, const size_t* sizes, int n,
                   uint32_t unit, hipStream_t stream, CachedCopy** result) {
+  int device = 0;
+  HVDHIP_CHECK(hipGetDevice(&device));
   std::vector<uint64_t> key;
   key.reserve(2 + 3 * (size_t)n);
-  key.push_back(unit);
+  key.push_back(((uint64_t)(uint32_t)device << 32) | unit);  // tables live on the device that built them
   key.push_back((uint64_t)n);
   for (int i = 0; i < n; ++i) {
     key.push_back((uint64_t)(uintptr_t)out[i]);
