@@ -14,13 +14,16 @@
 // triples in a fixed order and evaluates the coefficients.  No floating-point
 // atomics anywhere, so results are identical from run to run.
 // Pass 2 (scaled_add_k): one workgroup per chunk, a = ca*a + cb*b in double,
-// rounded once.
+// rounded once.  In the combine, when no layer has more than 512 triples, pass 2
+// does pass 1b's work itself (every workgroup re-adds its layer's triples in that
+// same fixed order under the shadow of its data loads) and pass 1b is not launched.
 //
 // Products of two fp32 (or fp16) values are exact in double, so only the
 // order of the double additions differs from the reference's sequential
 // loop.  Bandwidth-bound: 3 double fmas per 8 bytes read in pass 1.
 #include <cfloat>
 #include <cmath>
+#include <cstdlib>
 #include <list>
 #include <mutex>
 
@@ -136,6 +139,14 @@ __global__ __launch_bounds__(kWG) void dot_partials_k(const Chunk* __restrict__ 
   }
 }
 
+// Coefficients of adasum.h:397-404 from a layer's sums.
+__device__ __forceinline__ void layer_coeffs(const Triple& r, double guard, double* ca, double* cb) {
+  *ca = 1.;
+  *cb = 1.;
+  if (r.a >= guard) *ca = 1.0 - r.d / r.a * 0.5;
+  if (r.b >= guard) *cb = 1.0 - r.d / r.b * 0.5;
+}
+
 // One workgroup per layer: sums the layer's partial triples in a fixed order,
 // stores {dot, |a|^2, |b|^2} and the coefficients of adasum.h:397-404.
 __global__ __launch_bounds__(kWG) void finalize_k(const Layer* __restrict__ layers,
@@ -155,9 +166,8 @@ __global__ __launch_bounds__(kWG) void finalize_k(const Layer* __restrict__ laye
     normdots[3 * (uint64_t)blockIdx.x + 0] = r.d;
     normdots[3 * (uint64_t)blockIdx.x + 1] = r.a;
     normdots[3 * (uint64_t)blockIdx.x + 2] = r.b;
-    double ca = 1., cb = 1.;
-    if (r.a >= guard) ca = 1.0 - r.d / r.a * 0.5;
-    if (r.b >= guard) cb = 1.0 - r.d / r.b * 0.5;
+    double ca, cb;
+    layer_coeffs(r, guard, &ca, &cb);
     coeffs[2 * (uint64_t)blockIdx.x + 0] = ca;
     coeffs[2 * (uint64_t)blockIdx.x + 1] = cb;
   }
@@ -180,22 +190,100 @@ struct Axpby<half_t> {
   }
 };
 
-template <typename T>
+// FUSED = false: the coefficients come from `coeffs` (or, when that is null, from the
+// by-value pair).
+// FUSED = true (the combine, when no layer has more than 2*kWG partial triples): every
+// workgroup sums its layer's triples itself, in exactly the order finalize_k uses, while its
+// data loads are in flight, which saves the finalize launch between the two passes.  All
+// workgroups of a layer execute the same additions in the same order, so they agree to the
+// bit; the layer's first workgroup also stores the sums and coefficients for readers.
+template <typename T, bool FUSED>
 __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ chunks, T* a,
                                                     const T* __restrict__ b,
                                                     const double* __restrict__ coeffs,
-                                                    double ca_arg, double cb_arg) {
-  // coeffs == nullptr: every layer uses the by-value pair (ca_arg, cb_arg).
+                                                    double ca_arg, double cb_arg,
+                                                    const Layer* __restrict__ layers,
+                                                    const double* __restrict__ partials,
+                                                    double* __restrict__ normdots,
+                                                    double* __restrict__ coeffs_out, double guard,
+                                                    uint32_t nlayers) {
   constexpr int VEC = 16 / (int)sizeof(T);
   typedef Arr<T, VEC> V;
   const Chunk c = chunks[blockIdx.x];
-  const double ca = coeffs ? coeffs[2 * c.output] : ca_arg;
-  const double cb = coeffs ? coeffs[2 * c.output + 1] : cb_arg;
   const uint32_t n = c.n;
   gptr<T> pa = as_global(a + c.tensor);
   gptr<const T> pb = as_global(b + c.tensor);
   const uint32_t nv = n / VEC;
   uint32_t v = threadIdx.x;
+  double ca, cb;
+  if (FUSED) {
+    const Layer L = layers[c.output];
+    // this lane's share of the layer's triples first, the data loads behind them: loads return
+    // in order, so the sums below wait for the triples only
+    Triple t0 = {0., 0., 0.}, t1 = {0., 0., 0.};
+    if (threadIdx.x < L.count) {
+      const uint64_t i = 3 * ((uint64_t)L.first + threadIdx.x);
+      t0 = Triple{partials[i], partials[i + 1], partials[i + 2]};
+    }
+    if (threadIdx.x + kWG < L.count) {
+      const uint64_t i = 3 * ((uint64_t)L.first + threadIdx.x + kWG);
+      t1 = Triple{partials[i], partials[i + 1], partials[i + 2]};
+    }
+    const bool full = v + (kUnroll - 1) * kWG < nv;
+    V x[kUnroll], y[kUnroll];
+    if (full) {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        x[u] = ldv<T, VEC>(pa + (size_t)(v + u * kWG) * VEC);
+        y[u] = ldv<T, VEC>(pb + (size_t)(v + u * kWG) * VEC);
+      }
+    }
+    Triple t = {0., 0., 0.};
+    t.d += t0.d; t.a += t0.a; t.b += t0.b;  // the order of finalize_k: i = lane, lane + kWG
+    t.d += t1.d; t.a += t1.a; t.b += t1.b;
+    const Triple r = wg_reduce(t);
+    __shared__ double cc[2];
+    if (threadIdx.x == 0) {
+      layer_coeffs(r, guard, &ca, &cb);
+      cc[0] = ca;
+      cc[1] = cb;
+      if (blockIdx.x == L.first) {
+        normdots[3 * c.output + 0] = r.d;
+        normdots[3 * c.output + 1] = r.a;
+        normdots[3 * c.output + 2] = r.b;
+        coeffs_out[2 * c.output + 0] = ca;
+        coeffs_out[2 * c.output + 1] = cb;
+      }
+    }
+    if (blockIdx.x == 0) {
+      // layers without elements have no workgroup of their own: sums 0, coefficients 1
+      for (uint32_t l = threadIdx.x; l < nlayers; l += kWG) {
+        if (layers[l].count == 0) {
+          normdots[3 * (uint64_t)l + 0] = 0.;
+          normdots[3 * (uint64_t)l + 1] = 0.;
+          normdots[3 * (uint64_t)l + 2] = 0.;
+          coeffs_out[2 * (uint64_t)l + 0] = 1.;
+          coeffs_out[2 * (uint64_t)l + 1] = 1.;
+        }
+      }
+    }
+    __syncthreads();
+    ca = cc[0];
+    cb = cc[1];
+    if (full) {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) x[u].v[j] = Axpby<T>::f(ca, x[u].v[j], cb, y[u].v[j]);
+        stv<T, VEC>(pa + (size_t)(v + u * kWG) * VEC, x[u]);
+      }
+      v += kUnroll * kWG;
+    }
+  } else {
+    // coeffs == nullptr: every layer uses the by-value pair (ca_arg, cb_arg).
+    ca = coeffs ? coeffs[2 * c.output] : ca_arg;
+    cb = coeffs ? coeffs[2 * c.output + 1] : cb_arg;
+  }
   for (; v + (kUnroll - 1) * kWG < nv; v += kUnroll * kWG) {
     V x[kUnroll], y[kUnroll];
 #pragma unroll
@@ -231,6 +319,7 @@ struct hvdhip_adasum_plan {
   int dtype = 0;
   int device = 0;  // the device that holds the tables and results
   int64_t total = 0;
+  uint32_t max_layer_chunks = 0;
   DevTables tables;
   Layer* layers = nullptr;    // device, nlayers entries
   double* results = nullptr;  // one allocation: partials | normdots | coeffs | layer table
@@ -241,7 +330,9 @@ struct hvdhip_adasum_plan {
 
 namespace {
 
-int plan_dot_norms(hvdhip_adasum_plan* p, const void* a, const void* b, hipStream_t s) {
+// finalize = false leaves the partial triples for a fused scaled add to sum.
+int plan_dot_norms(hvdhip_adasum_plan* p, const void* a, const void* b, hipStream_t s,
+                   bool finalize = true) {
   if (p->nlayers == 0) return 0;
   const DevTables& t = p->tables;
   if (t.nchunks > 0) {
@@ -261,33 +352,50 @@ int plan_dot_norms(hvdhip_adasum_plan* p, const void* a, const void* b, hipStrea
     }
     HVDHIP_CHECK_LAUNCH("dot_partials_k");
   }
+  if (!finalize) return 0;
   hipLaunchKernelGGL(finalize_k, dim3((uint32_t)p->nlayers), dim3(kWG), 0, s, p->layers, p->partials,
                      p->normdots, p->coeffs, std::sqrt(DBL_MIN));
   HVDHIP_CHECK_LAUNCH("finalize_k");
   return 0;
 }
 
-// coeffs == nullptr selects the by-value pair (ca, cb) for every layer.
-int plan_scaled_add(hvdhip_adasum_plan* p, void* a, const void* b, const double* coeffs,
-                    double ca, double cb, hipStream_t s) {
+template <typename T, bool FUSED>
+void launch_scaled_add(hvdhip_adasum_plan* p, void* a, const void* b, const double* coeffs,
+                       double ca, double cb, hipStream_t s) {
   const DevTables& t = p->tables;
-  if (t.nchunks == 0) return 0;
+  hipLaunchKernelGGL((scaled_add_k<T, FUSED>), dim3(t.nchunks), dim3(kWG), 0, s, t.chunks,
+                     static_cast<T*>(a), static_cast<const T*>(b), coeffs, ca, cb, p->layers,
+                     p->partials, p->normdots, p->coeffs, std::sqrt(DBL_MIN), (uint32_t)p->nlayers);
+}
+
+template <bool FUSED>
+int scaled_add_by_dtype(hvdhip_adasum_plan* p, void* a, const void* b, const double* coeffs,
+                        double ca, double cb, hipStream_t s) {
+  if (p->tables.nchunks == 0) return 0;
   switch (p->dtype) {
-  case HVDHIP_FLOAT16:
-    hipLaunchKernelGGL((scaled_add_k<half_t>), dim3(t.nchunks), dim3(kWG), 0, s, t.chunks,
-                       static_cast<half_t*>(a), static_cast<const half_t*>(b), coeffs, ca, cb);
-    break;
-  case HVDHIP_FLOAT32:
-    hipLaunchKernelGGL((scaled_add_k<float>), dim3(t.nchunks), dim3(kWG), 0, s, t.chunks,
-                       static_cast<float*>(a), static_cast<const float*>(b), coeffs, ca, cb);
-    break;
-  default:
-    hipLaunchKernelGGL((scaled_add_k<double>), dim3(t.nchunks), dim3(kWG), 0, s, t.chunks,
-                       static_cast<double*>(a), static_cast<const double*>(b), coeffs, ca, cb);
-    break;
+  case HVDHIP_FLOAT16: launch_scaled_add<half_t, FUSED>(p, a, b, coeffs, ca, cb, s); break;
+  case HVDHIP_FLOAT32: launch_scaled_add<float, FUSED>(p, a, b, coeffs, ca, cb, s); break;
+  default: launch_scaled_add<double, FUSED>(p, a, b, coeffs, ca, cb, s); break;
   }
   HVDHIP_CHECK_LAUNCH("scaled_add_k");
   return 0;
+}
+
+// coeffs == nullptr selects the by-value pair (ca, cb) for every layer.
+int plan_scaled_add(hvdhip_adasum_plan* p, void* a, const void* b, const double* coeffs,
+                    double ca, double cb, hipStream_t s) {
+  return scaled_add_by_dtype<false>(p, a, b, coeffs, ca, cb, s);
+}
+
+// The combine may leave the layer sums to the scaled add when every layer's partial triples
+// fit the two loads per lane that kernel spends on them and there is a workgroup to do it.
+// HVDHIP_ADASUM_FUSED_COEFFS=0 keeps the separate finalize launch, for comparison.
+bool fused_coeffs_enabled() {
+  static const bool on = [] {
+    const char* e = std::getenv("HVDHIP_ADASUM_FUSED_COEFFS");
+    return !(e && e[0] == '0');
+  }();
+  return on;
 }
 
 int check_vectors(const hvdhip_adasum_plan* p, const void* a, const void* b) {
@@ -351,6 +459,7 @@ int hvdhip_adasum_plan_create(const int* tensor_counts, int nlayers, int dtype,
   std::vector<Layer> layers((size_t)nlayers);
   std::vector<Chunk> chunks;
   uint64_t off = 0;
+  uint32_t max_layer_chunks = 0;
   for (int i = 0; i < nlayers; ++i) {
     if (tensor_counts[i] < 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "tensor_counts[%d] is negative", i);
     const uint64_t n = (uint64_t)tensor_counts[i];
@@ -360,6 +469,7 @@ int hvdhip_adasum_plan_create(const int* tensor_counts, int nlayers, int dtype,
       chunks.push_back(Chunk{off + start, (uint64_t)i, 0, (uint32_t)(left < chunk_units ? left : chunk_units), 0});
     }
     layers[(size_t)i].count = (uint32_t)chunks.size() - layers[(size_t)i].first;
+    if (layers[(size_t)i].count > max_layer_chunks) max_layer_chunks = layers[(size_t)i].count;
     if (chunks.size() > kMaxWorkgroups) return fail(HVDHIP_ERR_TOO_LARGE, "the vectors need more than 2^23 workgroups");
     off += n;
   }
@@ -367,6 +477,7 @@ int hvdhip_adasum_plan_create(const int* tensor_counts, int nlayers, int dtype,
   p->nlayers = nlayers;
   p->dtype = dtype;
   p->total = (int64_t)off;
+  p->max_layer_chunks = max_layer_chunks;
   (void)hipGetDevice(&p->device);
   int rc = upload_chunks(chunks, &p->tables);
   if (rc) {
@@ -422,9 +533,12 @@ int hvdhip_adasum_combine(hvdhip_adasum_plan* plan, void* a, const void* b, void
   int rc = check_vectors(plan, a, b);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  rc = plan_dot_norms(plan, a, b, s);
+  const bool fused = plan->tables.nchunks > 0 && plan->max_layer_chunks <= 2 * (uint32_t)kWG &&
+                     fused_coeffs_enabled();
+  rc = plan_dot_norms(plan, a, b, s, !fused);
   if (rc) return rc;
-  rc = plan_scaled_add(plan, a, b, plan->coeffs, 0., 0., s);
+  rc = fused ? scaled_add_by_dtype<true>(plan, a, b, nullptr, 0., 0., s)
+             : plan_scaled_add(plan, a, b, plan->coeffs, 0., 0., s);
   return rc ? rc : ok();
 }
 

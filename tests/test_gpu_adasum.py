@@ -185,6 +185,43 @@ def test_results_are_reproducible_run_to_run(gpu):
     plan.destroy()
 
 
+@pytest.mark.parametrize("dtype", [F32, F64, F16])
+@pytest.mark.parametrize("big", [False, True])
+def test_combine_equals_split_sequence_bit_for_bit(gpu, dtype, big):
+    """combine() sums each layer's partial results inside the scaled add when every layer is
+    small enough, and launches the separate summing kernel otherwise (big: one layer beyond
+    that limit).  Both must give exactly what dot_norms() followed by scaled_add() gives:
+    same sums, same coefficients, same vector, to the bit, with empty layers reported as
+    sums 0 and coefficients 1."""
+    rng = np.random.default_rng(11)
+    np_t = NP_OF[dtype]
+    counts = [0, 5, 0, 70001, 16384 // SIZE_OF[dtype] * 512, 1, 0]  # fifth layer: exactly 512 chunks
+    if big:
+        counts[3] = 16384 // SIZE_OF[dtype] * 512 + 1  # 513 chunks
+    n = sum(counts)
+    a, b = _pair(rng, n, np_t)
+    d_a1, d_a2, d_b = gpu.upload(a), gpu.upload(a), gpu.upload(b)
+    plan1, plan2 = gpu.H.AdasumPlan(counts, dtype), gpu.H.AdasumPlan(counts, dtype)
+    try:
+        plan1.dot_norms(d_a1.data_ptr(), d_b.data_ptr(), gpu.stream)
+        plan1.scaled_add(d_a1.data_ptr(), d_b.data_ptr(), gpu.stream)
+        nd1, co1 = plan1.read(gpu.stream)
+        plan2.combine(d_a2.data_ptr(), d_b.data_ptr(), gpu.stream)
+        nd2, co2 = plan2.read(gpu.stream)
+        assert np.array_equal(np.array(nd1).view(np.uint64), np.array(nd2).view(np.uint64))
+        assert np.array_equal(np.array(co1).view(np.uint64), np.array(co2).view(np.uint64))
+        for i, c in enumerate(counts):
+            if c == 0:
+                assert list(nd2[3 * i:3 * i + 3]) == [0.0, 0.0, 0.0] and list(co2[2 * i:2 * i + 2]) == [1.0, 1.0]
+        raw = np.uint16 if np_t == np.float16 else np_t
+        g1, g2 = gpu.download(d_a1, raw), gpu.download(d_a2, raw)
+        assert np.array_equal(g1.view(np.uint8), g2.view(np.uint8))
+        assert not np.array_equal(g2.view(np.uint8), _raw(a).view(np.uint8)), "combine left the vector untouched"
+    finally:
+        plan1.destroy()
+        plan2.destroy()
+
+
 def test_rejects_integer_dtypes(gpu):
     import horovod_amd
     with pytest.raises(horovod_amd.HvdHipError) as e:
