@@ -36,6 +36,8 @@ _PV = POINTER(c_void_p)
 _PROTOTYPES = {
     "hvdhip_error_string": (c_char_p, [c_int]),
     "hvdhip_last_error": (c_char_p, []),
+    "hvdhip_set_fp16_scale_mode": (c_int, [c_int]),
+    "hvdhip_get_fp16_scale_mode": (c_int, []),
     "hvdhip_dtype_size": (c_int64, [c_int]),
     "hvdhip_get_device": (c_int, [POINTER(c_int)]),
     "hvdhip_set_device": (c_int, [c_int]),

@@ -6,6 +6,7 @@
 // timing-disabled events per (device, stream), filled with 128 events on
 // first use, guarded by a mutex because finalizer threads release events
 // while the background thread acquires them.
+#include <atomic>
 #include <cstdarg>
 #include <cstdlib>
 #include <cstring>
@@ -137,6 +138,15 @@ int free_tables(DevTables* t) {
   return 0;
 }
 
+std::atomic<int> g_fp16_scale_mode{HVDHIP_FP16_SCALE_FP32_FACTOR};
+
+float fp16_scale_factor(double scale) {
+  const float f = (float)scale;
+  if (g_fp16_scale_mode.load(std::memory_order_relaxed) == HVDHIP_FP16_SCALE_HALF_FACTOR)
+    return (float)(_Float16)f;  // __float2half((float)scale_factor), ops/cuda/cuda_kernels.cu:167
+  return f;
+}
+
 }  // namespace hvdhip
 
 using namespace hvdhip;
@@ -156,6 +166,15 @@ const char* hvdhip_error_string(int code) {
 }
 
 const char* hvdhip_last_error(void) { return g_last_error.c_str(); }
+
+int hvdhip_set_fp16_scale_mode(int mode) {
+  if (mode != HVDHIP_FP16_SCALE_FP32_FACTOR && mode != HVDHIP_FP16_SCALE_HALF_FACTOR)
+    return fail(HVDHIP_ERR_INVALID_ARGUMENT, "unknown fp16 scale mode %d", mode);
+  g_fp16_scale_mode.store(mode, std::memory_order_relaxed);
+  return ok();
+}
+
+int hvdhip_get_fp16_scale_mode(void) { return g_fp16_scale_mode.load(std::memory_order_relaxed); }
 
 int64_t hvdhip_dtype_size(int dtype) { return dtype_size(dtype); }
 

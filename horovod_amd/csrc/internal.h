@@ -49,6 +49,10 @@ inline int64_t dtype_size(int dtype) {
   }
 }
 
+// The fp32 factor that an fp16 scale multiplies by under the current fp16 scale mode:
+// (float)scale, or that value rounded to half (nearest even) and widened again.
+float fp16_scale_factor(double scale);
+
 // Threads per workgroup of every streaming kernel: four wave64 wavefronts.
 constexpr int kWG = 256;
 

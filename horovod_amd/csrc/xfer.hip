@@ -68,7 +68,9 @@ struct Scale {
 };
 
 // fp16 scaled through fp32 with an fp32 factor, one rounding to nearest even
-// (ops/collective_operations.h:99-127).
+// (ops/collective_operations.h:99-127).  When the host hands over a factor that a
+// half holds exactly, the fp32 product of two halves is exact and the result is the
+// correctly rounded half product, i.e. __hmul (ops/cuda/cuda_kernels.cu:96-136).
 struct ScaleHalf {
   typedef half_t S;
   typedef half_t D;
@@ -222,7 +224,7 @@ int launch_same_dtype(const DevTables& t, uint64_t base, double scale, int dtype
   case HVDHIP_INT8: return launch_xfer<Scale<int8_t, double>, MODE>(t, base, {scale}, stream);
   case HVDHIP_INT32: return launch_xfer<Scale<int32_t, double>, MODE>(t, base, {scale}, stream);
   case HVDHIP_INT64: return launch_xfer<Scale<int64_t, double>, MODE>(t, base, {scale}, stream);
-  case HVDHIP_FLOAT16: return launch_xfer<ScaleHalf, MODE>(t, base, {(float)scale}, stream);
+  case HVDHIP_FLOAT16: return launch_xfer<ScaleHalf, MODE>(t, base, {fp16_scale_factor(scale)}, stream);
   case HVDHIP_FLOAT32: return launch_xfer<Scale<float, float>, MODE>(t, base, {(float)scale}, stream);
   case HVDHIP_FLOAT64: return launch_xfer<Scale<double, double>, MODE>(t, base, {scale}, stream);
   default:
@@ -508,7 +510,7 @@ int hvdhip_scale_buffer(const void* fused_input_data, void* buffer_data, int64_t
   case HVDHIP_INT8: rc = launch_contig<Scale<int8_t, double>>(in, out, n, {scale_factor}, s); break;
   case HVDHIP_INT32: rc = launch_contig<Scale<int32_t, double>>(in, out, n, {scale_factor}, s); break;
   case HVDHIP_INT64: rc = launch_contig<Scale<int64_t, double>>(in, out, n, {scale_factor}, s); break;
-  case HVDHIP_FLOAT16: rc = launch_contig<ScaleHalf>(in, out, n, {(float)scale_factor}, s); break;
+  case HVDHIP_FLOAT16: rc = launch_contig<ScaleHalf>(in, out, n, {fp16_scale_factor(scale_factor)}, s); break;
   case HVDHIP_FLOAT32: rc = launch_contig<Scale<float, float>>(in, out, n, {(float)scale_factor}, s); break;
   default: rc = launch_contig<Scale<double, double>>(in, out, n, {scale_factor}, s); break;
   }
@@ -606,7 +608,7 @@ int hvdhip_fusion_pack(hvdhip_fusion_plan* plan, void* fusion_buffer, double sca
   int rc;
   if (plan->buffer_dtype != plan->tensor_dtype) {
     if (flags & HVDHIP_PACK_CAST_THEN_SCALE)
-      rc = launch_xfer<PackF32F16CastFirst, kPack>(plan->tables, base, {(float)scale_factor}, s);
+      rc = launch_xfer<PackF32F16CastFirst, kPack>(plan->tables, base, {fp16_scale_factor(scale_factor)}, s);
     else
       rc = launch_xfer<PackF32F16, kPack>(plan->tables, base, {(float)scale_factor}, s);
   } else {
@@ -627,7 +629,7 @@ int hvdhip_fusion_unpack(hvdhip_fusion_plan* plan, const void* fusion_buffer,
   const uint64_t base = (uint64_t)(uintptr_t)fusion_buffer;
   int rc;
   if (plan->buffer_dtype != plan->tensor_dtype) {
-    rc = launch_xfer<UnpackF16F32, kUnpack>(plan->unpack_tables, base, {(float)scale_factor}, s);
+    rc = launch_xfer<UnpackF16F32, kUnpack>(plan->unpack_tables, base, {fp16_scale_factor(scale_factor)}, s);
   } else {
     if (scale_factor != 1.0 && !scalable(plan->tensor_dtype))
       return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE, "dtype %d cannot be scaled", plan->tensor_dtype);

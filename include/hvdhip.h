@@ -64,6 +64,18 @@ enum hvdhip_dtype {
  * scale in fp32, then one rounding to half. */
 #define HVDHIP_PACK_CAST_THEN_SCALE 1u
 
+/* How an fp16 buffer is scaled (hvdhip_set_fp16_scale_mode()).  The reference has two
+ * arithmetics for it.  Its CPU path (ScaleBufferCPUImpl<unsigned short, float>,
+ * ops/collective_operations.h:99-127) widens the element to fp32, multiplies by
+ * (float)scale_factor and rounds once to half.  Its CUDA kernels
+ * (ops/cuda/cuda_kernels.cu:96-136,167-168,306-309) first round the factor to half,
+ * __float2half((float)scale_factor), and multiply half by half with one rounding.  The
+ * two agree for factors a half holds exactly (1/8, 0.5, 2 ...) and differ in the last
+ * bit of some elements otherwise; test/parallel/test_torch.py:339-445 expects the
+ * first for host tensors and the second for device tensors. */
+#define HVDHIP_FP16_SCALE_FP32_FACTOR 0 /* default: the CPU path's arithmetic */
+#define HVDHIP_FP16_SCALE_HALF_FACTOR 1 /* the CUDA kernels' arithmetic */
+
 /* Kinds for hvdhip_memcpy_async(). */
 #define HVDHIP_MEMCPY_H2D 1
 #define HVDHIP_MEMCPY_D2H 2
@@ -80,6 +92,16 @@ const char* hvdhip_error_string(int code);
 
 /* Detail of the calling thread's most recent failure ("" if none). */
 const char* hvdhip_last_error(void);
+
+/* Selects the arithmetic of every later fp16 scale in this process (scale_buffer, the
+ * scaled batched copy, pack and unpack of FLOAT16 plans, the cast-then-scale pack and the
+ * postscale of the unpack of converting plans): one of HVDHIP_FP16_SCALE_*.  The factor is
+ * prepared on the host when a call is made, so calls already queued are not affected.  The
+ * fused scale-then-cast pack of converting plans has no counterpart in the reference and
+ * always multiplies in fp32 by (float)scale_factor.  hvdhip_get_fp16_scale_mode() returns
+ * the current mode. */
+int hvdhip_set_fp16_scale_mode(int mode);
+int hvdhip_get_fp16_scale_mode(void);
 
 /* Size in bytes of one element, DataType_Size (common/message.cc:66-92); -1 if unknown. */
 int64_t hvdhip_dtype_size(int dtype);
@@ -168,8 +190,10 @@ int hvdhip_batched_scaled_d2d_memcpy(void* const* out, const void* const* in,
  * Arithmetic is that of ScaleBufferCPUImpl (ops/collective_operations.h:91-127):
  * u8/i8/i32/i64/f64 multiply in double and convert back (integers truncate
  * toward zero), f32 multiplies by (float)scale_factor, f16 converts to fp32,
- * multiplies by (float)scale_factor and rounds to nearest even.  Other dtypes
- * return HVDHIP_ERR_UNSUPPORTED_DTYPE. */
+ * multiplies by (float)scale_factor and rounds to nearest even (or, under
+ * HVDHIP_FP16_SCALE_HALF_FACTOR, by the factor rounded to half, which is the
+ * arithmetic of ScaleBufferCudaImpl itself).  Other dtypes return
+ * HVDHIP_ERR_UNSUPPORTED_DTYPE. */
 int hvdhip_scale_buffer(const void* fused_input_data, void* buffer_data, int64_t num_elements,
                         double scale_factor, int dtype, void* stream);
 

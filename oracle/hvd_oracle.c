@@ -23,6 +23,10 @@
  *       round trip identity, byte-pattern tensors (no cross-tensor bleed).
  *   orc_scale_buffer                 IEEE closed forms in numpy: one fp32 or
  *       fp64 product; trunc-toward-zero for integers; fp16 through fp32.
+ *   orc_scale_half_cuda              numpy float16 product (exact product of two
+ *       halves, one rounding) with the factor rounded to float16 first, on every
+ *       half bit pattern; the expectation test/parallel/test_torch.py:339-445
+ *       computes for device half tensors (factor.type(half) * tensor.type(half)).
  *   orc_sum                          numpy elementwise add per dtype.
  *   orc_adasum_dot_norms             math.fsum / numpy float64 dot.
  *   orc_adasum_coeffs, _scaled_add,  the numpy restatement held by the
@@ -215,6 +219,19 @@ void orc_scale_half_scalar(const uint16_t* in, uint16_t* out, int64_t n, float f
     float p = factor * half_bits_to_float(in[i]);
     out[i] = float_to_half_bits(p);
   }
+}
+
+/* The fp16 scale of the reference's CUDA kernels, ops/cuda/cuda_kernels.cu:96-136 with
+ * the factor prepared at :167 (and :306-309 for the batched scaled copy): the factor is
+ * rounded to half first, __float2half((float)scale_factor), then half times half with one
+ * rounding.  The kernels' own branch for devices without half arithmetic (:115-118,
+ * :131-134) spells the same value as
+ * __float2half(__half2float(scale_factor) * __half2float(input[i])), which is what this
+ * restates with the software converters: the fp32 product of two halves is exact. */
+void orc_scale_half_cuda(const uint16_t* in, uint16_t* out, int64_t n, double scale) {
+  const uint16_t hs = float_to_half_bits((float)scale);
+  const float fs = half_bits_to_float(hs);
+  for (int64_t i = 0; i < n; ++i) out[i] = float_to_half_bits(fs * half_bits_to_float(in[i]));
 }
 
 #define SCALE_LOOP(T, TS)                                                     \

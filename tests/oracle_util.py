@@ -129,6 +129,12 @@ class Oracle:
         self.lib.orc_scale_half_scalar(_p(h), _p(out), c_int64(h.size), c_float(factor))
         return out
 
+    def scale_half_cuda(self, h, scale):
+        h = np.ascontiguousarray(h, np.uint16)
+        out = np.empty_like(h)
+        self.lib.orc_scale_half_cuda(_p(h), _p(out), c_int64(h.size), c_double(scale))
+        return out
+
     def scale_cast_f32_to_f16(self, x, scale, cast_first=False):
         x = np.ascontiguousarray(x, np.float32)
         out = np.empty(x.shape, np.uint16)

@@ -53,6 +53,39 @@ def test_scale_f16_goes_through_fp32_with_fp32_factor(orc, factor):
         assert np.array_equal(orc.scale_buffer(h[:n], factor, F16), want[:n])
 
 
+@pytest.mark.parametrize("factor", FACTORS + [0.1915194503788923])
+def test_scale_f16_cuda_arithmetic_rounds_the_factor_to_half_first(orc, factor):
+    """ops/cuda/cuda_kernels.cu:96-136,167: half(factor) * x in half arithmetic.  numpy's
+    float16 product is the exact product rounded once, like __hmul."""
+    h = np.arange(65536, dtype=np.uint16)
+    h = h[~np.isnan(h.view(np.float16))]
+    with np.errstate(over="ignore"):
+        want = (np.float16(np.float32(factor)) * h.view(np.float16)).view(np.uint16)
+    got = orc.scale_half_cuda(h, factor)
+    assert np.array_equal(got, want)
+    if float(np.float16(np.float32(factor))) == factor:
+        # a factor that a half holds exactly: both arithmetics of the reference agree
+        assert np.array_equal(got, orc.scale_buffer(h, factor, F16))
+    else:
+        assert not np.array_equal(got, orc.scale_buffer(h, factor, F16))
+
+
+def test_scale_f16_cuda_arithmetic_on_the_reference_test_vector(orc):
+    """test/parallel/test_torch.py:339-388 for device half tensors: integers in [-100, 100)
+    times np.random.seed(1234); np.random.uniform(), expected as
+    (factor.type(half) * tensor.type(half)); for host half tensors the expectation is the
+    fp32 product rounded to half."""
+    np.random.seed(1234)
+    factor = np.random.uniform()
+    assert factor == 0.1915194503788923
+    x = np.arange(-100, 100).astype(np.float16)
+    want_device = np.float16(factor) * x
+    want_host = (np.float32(factor) * x.astype(np.float32)).astype(np.float16)
+    assert np.array_equal(orc.scale_half_cuda(x.view(np.uint16), factor), want_device.view(np.uint16))
+    assert np.array_equal(orc.scale_buffer(x.view(np.uint16), factor, F16), want_host.view(np.uint16))
+    assert not np.array_equal(want_device, want_host)  # the two expectations really differ on this vector
+
+
 @pytest.mark.parametrize("dtype", [U16, I16, BOOL])
 def test_scale_rejects_types_the_reference_rejects(orc, dtype):
     with pytest.raises(ValueError):
