@@ -110,6 +110,27 @@ def lib():
     return _lib
 
 
+_adapter = None
+
+
+def adapter_lib():
+    """libhvdhip_adapter.so: the C++ mirror of the reference's op-layer classes, with the
+    plain-C surface the Python callers use (keyed response fusion among others)."""
+    global _adapter
+    if _adapter is not None:
+        return _adapter
+    lib()  # the adapter links libhvdhip.so; load that one (and torch's HIP runtime) first
+    path = os.path.join(_HERE, "lib", "libhvdhip_adapter.so")
+    if not os.path.exists(path):
+        raise RuntimeError("%s is missing: build it with `make -C horovod_amd/csrc`; "
+                           "there is no fallback path" % path)
+    cdll = ctypes.CDLL(path)
+    cdll.hvd_adapter_fuse_keyed.restype = c_int
+    cdll.hvd_adapter_fuse_keyed.argtypes = [POINTER(c_int64), POINTER(c_int), c_int, c_int64, c_int, POINTER(c_int)]
+    _adapter = cdll
+    return _adapter
+
+
 def check(code, what):
     if code != 0:
         L = lib()

@@ -187,4 +187,15 @@ int hvd_adapter_fuse(const int64_t* tensor_bytes, int n, int64_t threshold, int 
   return (int)groups.size();
 }
 
+// keys[i]: an opaque class of responses that may fuse with each other.
+int hvd_adapter_fuse_keyed(const int64_t* tensor_bytes, const int* keys, int n, int64_t threshold,
+                           int batch_d2d_memcopies, int* group_of) {
+  std::vector<int64_t> tb(tensor_bytes, tensor_bytes + n);
+  std::vector<int> k(keys, keys + n);
+  auto groups = FuseResponses(tb, k, threshold, batch_d2d_memcopies != 0);
+  for (size_t g = 0; g < groups.size(); ++g)
+    for (int i : groups[g]) group_of[i] = (int)g;
+  return (int)groups.size();
+}
+
 }  // extern "C"

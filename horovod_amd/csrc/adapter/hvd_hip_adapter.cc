@@ -451,6 +451,13 @@ void AdasumGPU::FusedPairwiseReduce(void* a, const void* b, DataType horovod_dat
 
 std::vector<std::vector<int>> FuseResponses(const std::vector<int64_t>& tensor_bytes,
                                             int64_t fusion_threshold_bytes, bool batch_d2d_memcopies) {
+  return FuseResponses(tensor_bytes, std::vector<int>(tensor_bytes.size(), 0), fusion_threshold_bytes,
+                       batch_d2d_memcopies);
+}
+
+std::vector<std::vector<int>> FuseResponses(const std::vector<int64_t>& tensor_bytes,
+                                            const std::vector<int>& keys, int64_t fusion_threshold_bytes,
+                                            bool batch_d2d_memcopies) {
   auto padded = [&](int64_t s) { return batch_d2d_memcopies ? 16 * ((s + 15) / 16) : s; };
   const int n = (int)tensor_bytes.size();
   std::vector<int> group_of((size_t)n, -1);
@@ -465,11 +472,13 @@ std::vector<std::vector<int>> FuseResponses(const std::vector<int64_t>& tensor_b
     for (int j = head + 1; j < n; ++j) {
       if (group_of[(size_t)j] != -1) continue;
       const int64_t new_tensor_size = padded(tensor_bytes[(size_t)j]);
-      if (tensor_size + new_tensor_size <= fusion_threshold_bytes) {
+      if (keys[(size_t)j] == keys[(size_t)head] && tensor_size + new_tensor_size <= fusion_threshold_bytes) {
         tensor_size += new_tensor_size;
         group_of[(size_t)j] = g;
         groups[(size_t)g].push_back(j);
       } else {
+        // look ahead past a response that does not fit or does not match, while the batch
+        // plus everything skipped still fits (common/controller.cc:839-856)
         skipped_size += new_tensor_size;
         if (tensor_size + skipped_size > fusion_threshold_bytes) break;
       }

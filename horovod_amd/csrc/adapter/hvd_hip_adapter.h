@@ -227,6 +227,12 @@ private:
 // dtype and one pair of scale factors: returns groups of entry indices.
 std::vector<std::vector<int>> FuseResponses(const std::vector<int64_t>& tensor_bytes,
                                             int64_t fusion_threshold_bytes, bool batch_d2d_memcopies);
+// The same with mixed responses: keys[i] stands for everything that has to be equal for two
+// responses to fuse (response type, devices, dtype, prescale and postscale factor,
+// common/controller.cc:831-836); responses with different keys never share a group.
+std::vector<std::vector<int>> FuseResponses(const std::vector<int64_t>& tensor_bytes,
+                                            const std::vector<int>& keys, int64_t fusion_threshold_bytes,
+                                            bool batch_d2d_memcopies);
 
 }  // namespace common
 }  // namespace horovod

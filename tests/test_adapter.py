@@ -19,7 +19,8 @@ def _load():
 def test_adapter_loads_and_exports_its_test_surface():
     lib = _load()
     for name in ("hvd_adapter_create", "hvd_adapter_destroy", "hvd_adapter_allreduce", "hvd_adapter_state",
-                 "hvd_adapter_adasum_pairwise", "hvd_adapter_adasum_dispatch", "hvd_adapter_fuse"):
+                 "hvd_adapter_adasum_pairwise", "hvd_adapter_adasum_dispatch", "hvd_adapter_fuse",
+                 "hvd_adapter_fuse_keyed"):
         assert hasattr(lib, name)
 
 
@@ -36,6 +37,26 @@ def test_fuse_responses_matches_the_oracle(orc):
                                      ctypes.c_void_p(groups.ctypes.data))
         want_n, want = orc.fuse_responses(sizes, thr, pad16=bool(pad))
         assert got_n == want_n and np.array_equal(groups, want)
+
+
+def test_fuse_responses_with_mixed_keys_matches_the_oracle(orc):
+    """Mixed-precision queues: responses of another dtype or with other scale factors are
+    looked past, not fused (common/controller.cc:831-856)."""
+    lib = _load()
+    rng = np.random.default_rng(32)
+    for trial in range(300):
+        n = int(rng.integers(1, 60))
+        sizes = rng.integers(1, 400, n).astype(np.int64)
+        keys = rng.integers(0, int(rng.integers(1, 4)), n).astype(np.int32)
+        thr = int(rng.integers(50, 1200))
+        pad = trial % 2
+        groups = np.full(n, -1, np.int32)
+        got_n = lib.hvd_adapter_fuse_keyed(ctypes.c_void_p(sizes.ctypes.data), ctypes.c_void_p(keys.ctypes.data), n,
+                                           ctypes.c_int64(thr), pad, ctypes.c_void_p(groups.ctypes.data))
+        want_n, want = orc.fuse_responses(sizes, thr, pad16=bool(pad), keys=keys)
+        assert got_n == want_n and np.array_equal(groups, want)
+        for g in range(got_n):
+            assert len(set(keys[groups == g])) == 1
 
 
 def test_python_planner_matches_the_oracle(orc):

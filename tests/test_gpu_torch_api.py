@@ -1,0 +1,314 @@
+"""The allreduce surface of horovod.torch in front of the HIP path.
+
+The first half restates the reference's own tests (test/parallel/test_torch.py:152-445,
+607-705 and 1340-1400) for a simulated world: same inputs (integers in [-100, 100) in 17,
+17x17 and 17x17x17 tensors, every rank holding the same values), same expectations.  The
+second half gives every rank its own values and checks against the CPU oracle."""
+import itertools
+import warnings
+
+import numpy as np
+import pytest
+import torch
+
+from oracle_util import F16, F32, F64
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.int32, torch.int64, torch.float32, torch.float64, torch.float16]
+INT_TYPES = [torch.int32, torch.int64]
+DIMS = [1, 2, 3]
+
+
+@pytest.fixture()
+def hvd(gpu):
+    import horovod_amd.torch as hvd
+    yield hvd
+    hvd.shutdown()
+    gpu.H.set_fp16_scale_mode(gpu.H.FP16_SCALE_FP32_FACTOR)
+
+
+def _tensor(dtype, dim, seed=1234):
+    torch.manual_seed(seed)
+    return torch.FloatTensor(*([17] * dim)).random_(-100, 100).cuda().type(dtype)
+
+
+@pytest.mark.parametrize("size", [1, 2, 3, 8])
+def test_horovod_allreduce(hvd, size):
+    """test_torch.py:152-183: the sum over ranks holding equal tensors is tensor * size."""
+    hvd.init(size=size)
+    for dtype, dim in itertools.product(DTYPES, DIMS):
+        tensor = _tensor(dtype, dim)
+        summed = hvd.allreduce(tensor, average=False)
+        assert torch.equal(summed, tensor * size), (dtype, dim)
+        assert summed.data_ptr() != tensor.data_ptr()
+
+
+@pytest.mark.parametrize("size", [1, 2, 4])
+def test_horovod_allreduce_average(hvd, size):
+    """test_torch.py:185-216: Average gives the tensor back (exactly, for a power-of-two size)."""
+    hvd.init(size=size)
+    for dtype, dim in itertools.product(DTYPES, DIMS):
+        tensor = _tensor(dtype, dim)
+        averaged = hvd.allreduce(tensor, average=True)
+        assert torch.equal(averaged, tensor), (dtype, dim)
+        assert torch.equal(hvd.allreduce(tensor), tensor)  # Average is the default op
+        assert torch.equal(hvd.allreduce(tensor, op=hvd.Average), tensor)
+
+
+def test_horovod_allreduce_average_three_ranks_within_threshold(hvd):
+    hvd.init(size=3)
+    for dtype in (torch.float32, torch.float64, torch.float16):
+        tensor = _tensor(dtype, 2)
+        assert torch.allclose(hvd.allreduce(tensor, average=True), tensor, 1e-3 if dtype == torch.float16 else 1e-6)
+
+
+@pytest.mark.parametrize("size", [1, 2])
+def test_horovod_allreduce_inplace_and_async_fused(hvd, size):
+    """test_torch.py:218-297: in place; many requests in flight are fused into few responses."""
+    hvd.init(size=size)
+    for dtype, dim in itertools.product(DTYPES, DIMS):
+        tensor = _tensor(dtype, dim)
+        want = tensor * size
+        hvd.allreduce_(tensor, average=False)
+        assert torch.equal(tensor, want)
+    import horovod_amd.torch.mpi_ops as ops
+    before = ops._engine.responses
+    tests = []
+    for dtype, dim in itertools.product(DTYPES, DIMS):
+        tensor = _tensor(dtype, dim)
+        tests.append((tensor * size, hvd.allreduce_async(tensor, average=False)))
+    polled = [hvd.poll(h) for _, h in tests]
+    assert all(isinstance(p, bool) for p in polled)
+    for want, handle in tests:
+        assert torch.equal(hvd.synchronize(handle), want)
+    # 15 requests of 5 dtypes: one fused response per dtype
+    assert ops._engine.responses - before == len(DTYPES)
+
+
+def _expected_scaled(tensor, factor, dtype, half_factor_mode):
+    """The expectation of test_torch.py:363-375 / :418-431: integers scale in float64; device
+    half tensors in half arithmetic with the factor rounded to half, host half tensors in
+    float32 with the float32 factor."""
+    if dtype in INT_TYPES:
+        return (torch.tensor(factor, dtype=torch.float64) * tensor.cpu().type(torch.float64))
+    if dtype == torch.float16 and not half_factor_mode:
+        return torch.tensor(factor, dtype=torch.float32) * tensor.cpu().type(torch.float32)
+    return torch.tensor(factor, dtype=torch.float64).type(dtype) * tensor.cpu()
+
+
+@pytest.mark.parametrize("half_factor_mode", [False, True])
+@pytest.mark.parametrize("size", [1, 2])
+def test_horovod_allreduce_prescale(hvd, gpu, size, half_factor_mode):
+    """test_torch.py:339-388."""
+    hvd.init(size=size)
+    if half_factor_mode:
+        gpu.H.set_fp16_scale_mode(gpu.H.FP16_SCALE_HALF_FACTOR)
+    for dtype, dim in itertools.product(DTYPES, DIMS):
+        np.random.seed(1234)
+        factor = np.random.uniform()
+        tensor = _tensor(dtype, dim)
+        summed = hvd.allreduce(tensor, average=False, prescale_factor=factor)
+        multiplied = _expected_scaled(tensor, factor, dtype, half_factor_mode).type(dtype) * size
+        assert torch.equal(summed.cpu(), multiplied), (dtype, dim)
+
+
+@pytest.mark.parametrize("half_factor_mode", [False, True])
+@pytest.mark.parametrize("size", [1, 2])
+def test_horovod_allreduce_postscale(hvd, gpu, size, half_factor_mode):
+    """test_torch.py:390-445."""
+    hvd.init(size=size)
+    if half_factor_mode:
+        gpu.H.set_fp16_scale_mode(gpu.H.FP16_SCALE_HALF_FACTOR)
+    for dtype, dim in itertools.product(DTYPES, DIMS):
+        np.random.seed(1234)
+        factor = np.random.uniform()
+        tensor = _tensor(dtype, dim)
+        summed = hvd.allreduce(tensor, average=False, postscale_factor=factor)
+        multiplied = _expected_scaled(tensor * size, factor, dtype, half_factor_mode).type(dtype)
+        assert torch.equal(summed.cpu(), multiplied), (dtype, dim)
+
+
+@pytest.mark.parametrize("size", [1, 2, 4])
+def test_horovod_grouped_allreduce(hvd, size):
+    """test_torch.py:607-705: sum, average and in place, five tensors per group."""
+    hvd.init(size=size)
+    import horovod_amd.torch.mpi_ops as ops
+    for dtype, dim in itertools.product(DTYPES, DIMS):
+        torch.manual_seed(1234)
+        tensors = [torch.FloatTensor(*([17] * dim)).random_(-100, 100).cuda().type(dtype) for _ in range(5)]
+        before = ops._engine.responses
+        summed = hvd.grouped_allreduce(tensors, average=False)
+        assert ops._engine.responses - before == 1  # the group travels as one fused response
+        assert all(torch.equal(s, t * size) for s, t in zip(summed, tensors))
+        averaged = hvd.grouped_allreduce(tensors, average=True)
+        assert all(torch.equal(a, t) for a, t in zip(averaged, tensors))
+        want = [t * size for t in tensors]
+        hvd.grouped_allreduce_(tensors, average=False)
+        assert all(torch.equal(t, w) for t, w in zip(tensors, want))
+
+
+def test_horovod_allreduce_grad(hvd):
+    """test_torch.py:547-605: the gradient of a sum over ranks is ones * size; of an average, ones."""
+    hvd.init(size=4)
+    for dtype, dim in itertools.product([torch.float32, torch.float64, torch.float16], DIMS):
+        tensor = _tensor(dtype, dim)
+        tensor.requires_grad_()
+        summed = hvd.allreduce(tensor, average=False)
+        summed.backward(torch.ones([17] * dim, device="cuda", dtype=dtype))
+        assert torch.equal(tensor.grad, torch.ones([17] * dim, device="cuda", dtype=dtype) * 4)
+        tensor.grad = None
+        hvd.allreduce(tensor, average=True).backward(torch.ones([17] * dim, device="cuda", dtype=dtype))
+        assert torch.equal(tensor.grad, torch.ones([17] * dim, device="cuda", dtype=dtype))
+
+
+def test_errors_of_the_front_end(hvd):
+    with pytest.raises(ValueError, match="not been initialized"):
+        hvd.size()
+    hvd.init(size=2)
+    t = torch.ones(8, device="cuda")
+    with pytest.raises(ValueError, match="supersedes average"):
+        hvd.allreduce(t, average=True, op=hvd.Sum)
+    with pytest.raises(ValueError, match="contiguous"):
+        hvd.allreduce_async_(torch.ones(4, 4, device="cuda").t())
+    with pytest.raises(ValueError, match="not supported"):
+        hvd.allreduce_async_(torch.ones(4))
+    with pytest.raises(ValueError, match="not supported"):
+        hvd.allreduce_async_(torch.ones(4, device="cuda", dtype=torch.complex64))
+    # test_torch.py:1340-1370: one name, two requests in flight
+    h = hvd.allreduce_async(t, name="duplicate_name")
+    with pytest.raises(hvd.HorovodInternalError, match="same name"):
+        hvd.allreduce_async(t, name="duplicate_name")
+    hvd.synchronize(h)
+    hvd.synchronize(hvd.allreduce_async(t, name="duplicate_name"))  # free again once synchronised
+    with pytest.raises(ValueError, match="Adasum"):
+        hvd.allreduce(torch.ones(4, device="cuda", dtype=torch.int32), op=hvd.Adasum)
+    with pytest.raises(ValueError, match="handle"):
+        hvd.poll(12345)
+    with warnings.catch_warnings(record=True) as w:
+        warnings.simplefilter("always")
+        hvd.allreduce(t, average=False)
+    assert any(issubclass(x.category, DeprecationWarning) for x in w)
+    hvd.shutdown()
+    hvd.init(size=6, local_size=2)
+    with pytest.raises(NotImplementedError, match="power of 2"):
+        hvd.allreduce(t, op=hvd.Adasum)
+
+
+# ---- every rank with values of its own, against the oracle --------------------------
+
+def _peer_values(rank, name, tensor):
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1000 * rank + sum(name.encode()) % 997)
+    if tensor.dtype.is_floating_point:
+        return torch.randn(tensor.shape, generator=g, device="cuda", dtype=torch.float32).type(tensor.dtype)
+    return torch.randint(-1000, 1000, tensor.shape, generator=g, device="cuda").type(tensor.dtype)
+
+
+def _np(t):
+    t = t.detach().cpu()
+    return t.view(torch.int16).numpy().view(np.uint16) if t.dtype == torch.float16 else t.numpy()
+
+
+@pytest.mark.parametrize("dtype,code", [(torch.float32, F32), (torch.float16, F16), (torch.float64, F64)])
+def test_sum_of_distinct_ranks_with_both_scale_factors(hvd, orc, dtype, code):
+    size = 8
+    hvd.init(size=size, peer_source=_peer_values)
+    torch.manual_seed(7)
+    shapes = [(5,), (300, 7), (1,), (64, 64, 3), (17,)]
+    tensors = [torch.randn(s, device="cuda").type(dtype) for s in shapes]
+    names = ["grad.%d" % i for i in range(len(tensors))]
+    pre, post = 0.125, 1.0 / 3.0
+    handles = [hvd.allreduce_async(t, op=hvd.Sum, name=n, prescale_factor=pre, postscale_factor=post)
+               for t, n in zip(tensors, names)]
+    outs = [hvd.synchronize(h) for h in handles]
+    for t, n, out in zip(tensors, names, outs):
+        acc = orc.scale_buffer(_np(t).reshape(-1), pre, code)
+        for rank in range(1, size):
+            peer = orc.scale_buffer(_np(_peer_values(rank, "allreduce." + n, t)).reshape(-1), pre, code)
+            acc = orc.sum(peer, acc, code)
+        want = orc.scale_buffer(acc, post, code)
+        assert np.array_equal(_np(out).reshape(-1).view(np.uint8), want.view(np.uint8)), n
+
+
+def test_fp16_compression_rides_on_pack_and_unpack(hvd, orc):
+    """hvd.allreduce(..., compression=hvd.Compression.fp16) on float32: the reference casts,
+    scales and sums in half and casts back (compression.py:46-64); here the two casts happen
+    in the pack and unpack kernels with the same roundings and no half tensor exists."""
+    size = 4
+    hvd.init(size=size, peer_source=_peer_values)
+    torch.manual_seed(9)
+    tensors = [torch.randn(s, device="cuda") * 1e-3 for s in [(1000,), (33, 5), (1,)]]
+    outs = hvd.grouped_allreduce(tensors, op=hvd.Average, name="g", compression=hvd.Compression.fp16,
+                                 prescale_factor=0.5, postscale_factor=2.0)
+    for i, (t, out) in enumerate(zip(tensors, outs)):
+        assert out.dtype == torch.float32
+        name = "grouped_allreduce.g_%dof%d" % (i + 1, len(tensors))
+        acc = orc.scale_cast_f32_to_f16(_np(t).reshape(-1), 0.5, cast_first=True)
+        for rank in range(1, size):
+            peer = orc.scale_cast_f32_to_f16(_np(_peer_values(rank, name, t)).reshape(-1), 0.5, cast_first=True)
+            acc = orc.float16_sum(peer, acc)
+        want = orc.scale_cast_f16_to_f32(acc, 2.0 / size)
+        assert np.array_equal(_np(out).reshape(-1).view(np.uint32), want.view(np.uint32))
+    # the unfused route through the compressor's own casts gives the same values
+    for t, out in zip(tensors, outs):
+        h, ctx = hvd.Compression.fp16.compress(t)
+        assert h.dtype == torch.float16 and hvd.Compression.fp16.decompress(h, ctx).dtype == torch.float32
+
+
+@pytest.mark.parametrize("size,local_size", [(2, 1), (4, 1), (4, 2)])
+@pytest.mark.parametrize("dtype,code", [(torch.float32, F32), (torch.float16, F16)])
+def test_adasum_tree_matches_pairwise_oracle(hvd, orc, size, local_size, dtype, code):
+    hvd.init(size=size, local_size=local_size, peer_source=_peer_values)
+    torch.manual_seed(11)
+    tensors = [torch.randn(s, device="cuda").type(dtype) for s in [(4099,), (7, 3), (20000,)]]
+    outs = hvd.grouped_allreduce(tensors, op=hvd.Adasum, name="a")
+    for i, (t, out) in enumerate(zip(tensors, outs)):
+        name = "grouped_allreduce.a_%dof%d" % (i + 1, len(tensors))
+        ranks = [_np(t).reshape(-1)] + [_np(_peer_values(r, name, t)).reshape(-1) for r in range(1, size)]
+        nodes = []
+        for node in range(size // local_size):
+            acc = ranks[node * local_size]
+            for r in ranks[node * local_size + 1:(node + 1) * local_size]:
+                acc = orc.sum(r, acc, code)
+            nodes.append(acc)
+        d = 1
+        while d < len(nodes):
+            for j in range(0, len(nodes), 2 * d):
+                nodes[j] = orc.adasum_pairwise(nodes[j], nodes[j + d], [t.numel()], code)[0]
+            d *= 2
+        want = orc.scale_buffer(nodes[0], 1.0 / local_size, code) if local_size > 1 else nodes[0]
+        got = _np(out).reshape(-1)
+        if dtype == torch.float16:
+            assert np.array_equal(got, want)
+        else:
+            ulp = np.abs(got.view(np.int32).astype(np.int64) - want.view(np.int32).astype(np.int64))
+            assert ulp.max() <= 2 * (size // local_size - 1), ulp.max()  # <= 1 ulp per level that feeds the next
+
+
+def test_requests_with_mixed_dtypes_and_factors_fuse_by_class(hvd):
+    hvd.init(size=2)
+    import horovod_amd.torch.mpi_ops as ops
+    a = [torch.ones(100, device="cuda") * i for i in range(4)]
+    b = [torch.ones(50, device="cuda", dtype=torch.float16) * i for i in range(3)]
+    handles = []
+    for i in range(4):
+        handles.append(hvd.allreduce_async(a[i], op=hvd.Sum))
+        if i < 3:
+            handles.append(hvd.allreduce_async(b[i], op=hvd.Sum))
+    handles.append(hvd.allreduce_async(a[1], op=hvd.Sum, prescale_factor=0.5))
+    before = ops._engine.responses
+    outs = [hvd.synchronize(h) for h in handles]
+    assert ops._engine.responses - before == 3  # fp32, fp16, and fp32 with another prescale
+    assert torch.equal(outs[2], a[1] * 2) and torch.equal(outs[3], b[1] * 2) and torch.equal(outs[-1], a[1])
+
+
+def test_small_fusion_threshold_splits_responses_and_two_streams_alternate(hvd):
+    hvd.init(size=2, fusion_threshold=4096, num_streams=2)
+    import horovod_amd.torch.mpi_ops as ops
+    ts = [torch.full((600,), float(i), device="cuda") for i in range(6)]  # 2,400 bytes each: one per response
+    hs = [hvd.allreduce_async(t, op=hvd.Sum) for t in ts]
+    outs = [hvd.synchronize(h) for h in hs]
+    assert ops._engine.responses == 6
+    for i, o in enumerate(outs):
+        assert torch.equal(o, ts[i] * 2)
