@@ -54,7 +54,11 @@ inline int64_t dtype_size(int dtype) {
 float fp16_scale_factor(double scale);
 
 // Threads per workgroup of every streaming kernel: four wave64 wavefronts.
-constexpr int kWG = 256;
+#ifndef HVDHIP_WG
+#define HVDHIP_WG 256
+#endif
+constexpr int kWG = HVDHIP_WG;
+static_assert(kWG % 64 == 0 && kWG >= 64 && kWG <= 1024, "whole wave64 wavefronts");
 
 // A launch may not exceed 2^32 - 1 threads in x.  Contiguous kernels cover larger buffers
 // in slices of kMaxWorkgroups workgroups; a plan that needs more is refused.
