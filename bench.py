@@ -489,6 +489,30 @@ def main():
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline_stress(counts, host)
+    two_streams = None
+    if not args.no_extra:
+        # The same steps alternating over two streams (HOROVOD_NUM_NCCL_STREAMS=2, one fusion buffer per
+        # stream slot as in common/fusion_buffer_manager.cc): the start-up and drain of one step's kernels
+        # overlap the other's.  Reported beside the headline value, which stays single-stream.
+        try:
+            pair = [stream, Stream()]
+
+            def step2():
+                i = turn[0] = (turn[0] + 1) % len(plans)
+                plans[i].pack(fbs[i].data_ptr(), 0.125, pair[i % 2])
+                plans[i].unpack(fbs[i].data_ptr(), 1.0, pair[i % 2])
+
+            def sync2():
+                pair[0].synchronize()
+                pair[1].synchronize()
+
+            sec2 = timed(step2, sync2, args.steps, args.warmup)
+            two_streams = {"GB/s": round(4 * payload / sec2 / 1e9, 1),
+                           "frac_of_hbm_peak": round(4 * payload / sec2 / 1e9 / HBM_PEAK_GBS, 4),
+                           "ms_per_step": round(sec2 * 1e3, 5), "streams": 2}
+            pair[1].destroy()
+        except Exception as e:  # pragma: no cover
+            two_streams = {"error": "%s: %s" % (type(e).__name__, e)}
     comparator = None
     if not args.no_extra:
         try:
@@ -506,6 +530,7 @@ def main():
         except Exception as e:  # pragma: no cover
             result["extra"] = {"error": "%s: %s" % (type(e).__name__, e)}
         result["extra"]["fusion_stress_execute_vs_per_tensor_copies"] = comparator
+        result["extra"]["fusion_stress_two_streams"] = two_streams
         if not args.no_cpu and "error" not in result["extra"]:
             try:
                 for name, v in cpu_extras().items():
