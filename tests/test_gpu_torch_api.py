@@ -312,3 +312,66 @@ def test_small_fusion_threshold_splits_responses_and_two_streams_alternate(hvd):
     assert ops._engine.responses == 6
     for i, o in enumerate(outs):
         assert torch.equal(o, ts[i] * 2)
+
+
+_FUZZ_TYPES = [(torch.uint8, 0), (torch.int8, 1), (torch.int32, 4), (torch.int64, 5), (torch.float16, 6),
+               (torch.float32, 7), (torch.float64, 8)]
+
+
+def _fuzz_values(gen, n, dtype, rank):
+    if dtype.is_floating_point:
+        return (torch.randn(n, generator=gen, device="cuda") * 3).type(dtype)
+    hi = 6 if dtype in (torch.uint8, torch.int8) else 1000
+    lo = 0 if dtype == torch.uint8 else -hi
+    return torch.randint(lo, hi, (n,), generator=gen, device="cuda").type(dtype)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_fuzz_against_the_oracle(hvd, orc, seed):
+    """Random worlds, dtypes, sizes (zero included), element-aligned-only addresses, factors,
+    ops, in place and out of place, all in flight together: every output equals
+    postscale * (sum over ranks in rank order of prescale * x_rank) as the oracle computes it."""
+    rng = np.random.default_rng(100 + seed)
+    size = int(rng.choice([1, 2, 3, 5, 8]))
+    store = {}
+
+    def peer_source(rank, name, tensor):
+        return store[name][rank]
+
+    hvd.init(size=size, peer_source=peer_source, fusion_threshold=int(rng.choice([1 << 12, 1 << 16, 64 << 20])),
+             num_streams=int(rng.choice([1, 2])))
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    factors = [1.0, 0.5, 0.125, 1.0 / 3.0, 2.5]
+    jobs = []
+    for i in range(int(rng.integers(1, 14))):
+        dtype, code = _FUZZ_TYPES[int(rng.integers(0, len(_FUZZ_TYPES)))]
+        n = int(rng.choice([0, 1, 3, 17, 255, 1024, 1025, 4099, 20000]))
+        shift = int(rng.integers(0, 4))
+        ranks = []
+        for r in range(size):
+            base = _fuzz_values(gen, n + 4, dtype, r)
+            ranks.append(base[shift:shift + n])
+        name = "fuzz.%d" % i
+        store["allreduce." + name] = ranks
+        average = bool(rng.integers(0, 2)) and dtype.is_floating_point
+        pre = float(rng.choice(factors))
+        post = float(rng.choice(factors))
+        if not dtype.is_floating_point and dtype != torch.int64 and dtype != torch.int32:
+            pre = post = 1.0 if rng.integers(0, 2) else 0.5  # keep 8-bit results inside the type
+        inplace = bool(rng.integers(0, 2))
+        want = orc.scale_buffer(_np(ranks[0]), pre, code) if n else _np(ranks[0])
+        for r in range(1, size):
+            if n:
+                want = orc.sum(orc.scale_buffer(_np(ranks[r]), pre, code), want, code)
+        if n:
+            want = orc.scale_buffer(want, post / size if average else post, code)
+        op = hvd.Average if average else hvd.Sum
+        fn = hvd.allreduce_async_ if inplace else hvd.allreduce_async
+        handle = fn(ranks[0], name=name, op=op, prescale_factor=pre, postscale_factor=post)
+        jobs.append((name, handle, want, n))
+    for name, handle, want, n in jobs:
+        out = hvd.synchronize(handle)
+        assert out.numel() == n
+        if n:
+            assert np.array_equal(_np(out).reshape(-1).view(np.uint8), np.ascontiguousarray(want).view(np.uint8)), name
