@@ -54,14 +54,23 @@ class Request:
         self.entries = entries
         self.op, self.prescale, self.postscale, self.divisor = op, float(prescale), float(postscale), divisor
         self.tensor_dtype, self.wire_dtype, self.device = tensor_dtype, wire_dtype, device
-        self.ready = None        # torch.cuda.Event recorded on the framework's stream at enqueue
-        self.markers = []        # (Stream, event) per fused response that carries one of the entries
+        self.producer = None     # the framework stream that was current at enqueue
+        self.markers = []        # one Marker per fused response that carries one of the entries
         self.keepalive = []      # peer tensors in flight
         self.submitted = False
         self.error = None
 
     def key(self):
         return (self.op, self.device, self.tensor_dtype, self.wire_dtype, self.prescale, self.postscale)
+
+
+class Marker:
+    """Completion event of one fused response, shared by the requests it carried
+    (ops/gpu_operations.cc:50-56 records one per response)."""
+    __slots__ = ("stream", "event", "refs")
+
+    def __init__(self, stream, event, refs):
+        self.stream, self.event, self.refs = stream, event, refs
 
 
 class Engine:
@@ -82,6 +91,7 @@ class Engine:
         self.max_plans = max_plans
         self.cycles = 0
         self.responses = 0       # fused responses executed so far
+        self.ready = {}          # framework stream -> event recorded at the start of the current cycle
 
     # ---- queueing -------------------------------------------------------
 
@@ -95,8 +105,11 @@ class Engine:
                     "tensor name.")
         for e in request.entries:
             self.inflight[e.name] = request
-        request.ready = torch.cuda.Event()
-        request.ready.record()  # RecordReadyEvent, horovod/torch/ready_event.cc
+        # The reference records a ready event per request on the framework's stream
+        # (RecordReadyEvent, horovod/torch/ready_event.cc).  A cycle here runs on the caller's own
+        # thread, after every enqueue it serves, so one event per producing stream and cycle, recorded
+        # when the cycle starts, orders the same work and costs one record instead of one per tensor.
+        request.producer = torch.cuda.current_stream()
         self.queue.append(request)
 
     def run_cycle(self):
@@ -106,6 +119,12 @@ class Engine:
         if not pending:
             return
         self.cycles += 1
+        self.ready = {}
+        for r in pending:
+            if r.producer not in self.ready:
+                ev = torch.cuda.Event()
+                ev.record(r.producer)
+                self.ready[r.producer] = ev
         flat = [(r, e) for r in pending for e in r.entries]
         n = len(flat)
         sizes = (c_int64 * n)(*[e.count * dtype_size(r.wire_dtype) for r, e in flat])
@@ -180,8 +199,10 @@ class Engine:
         for r, _ in group:
             if r not in requests:
                 requests.append(r)
-        for r in requests:  # the op's stream waits for the framework's stream, ops/nccl_operations.cc:140-154
-            check(lib().hvdhip_stream_wait_event(s.handle, c_void_p(r.ready.cuda_event)), "hvdhip_stream_wait_event")
+        # the op's stream waits for the framework's stream(s), ops/nccl_operations.cc:140-154
+        for producer in {r.producer for r in requests}:
+            check(lib().hvdhip_stream_wait_event(s.handle, c_void_p(self.ready[producer].cuda_event)),
+                  "hvdhip_stream_wait_event")
         counts = [e.count for _, e in group]
         fused = len(group) > 1 or wire != tdt
         flags = PACK_CAST_THEN_SCALE if wire != tdt else 0
@@ -231,11 +252,12 @@ class Engine:
         elif first.postscale != 1.0 and nelem:
             H.scale_buffer(result, result, nelem, first.postscale, tdt, s)
 
-        for r in requests:  # completion marker from the event pool, ops/gpu_operations.cc:50-56
-            ev = c_void_p()
-            check(lib().hvdhip_event_acquire(s.handle, ctypes.byref(ev)), "hvdhip_event_acquire")
-            check(lib().hvdhip_event_record(ev, s.handle), "hvdhip_event_record")
-            r.markers.append((s, ev))
+        ev = c_void_p()  # completion marker from the event pool
+        check(lib().hvdhip_event_acquire(s.handle, ctypes.byref(ev)), "hvdhip_event_acquire")
+        check(lib().hvdhip_event_record(ev, s.handle), "hvdhip_event_record")
+        marker = Marker(s, ev, len(requests))
+        for r in requests:
+            r.markers.append(marker)
 
     @staticmethod
     def _scale_or_copy(src, dst, count, scale, dtype, s):
@@ -279,9 +301,9 @@ class Engine:
             self.run_cycle()
         if request.error is not None:
             return True
-        for _, ev in request.markers:
+        for m in request.markers:
             done = c_int()
-            check(lib().hvdhip_event_query(ev, ctypes.byref(done)), "hvdhip_event_query")
+            check(lib().hvdhip_event_query(m.event, ctypes.byref(done)), "hvdhip_event_query")
             if not done.value:
                 return False
         return True
@@ -290,10 +312,13 @@ class Engine:
         if not request.submitted:
             self.run_cycle()
         try:
-            for s, ev in request.markers:
-                check(lib().hvdhip_event_synchronize(ev), "hvdhip_event_synchronize")
-                check(lib().hvdhip_event_release(s.handle, ev), "hvdhip_event_release")
+            for m in request.markers:
+                check(lib().hvdhip_event_synchronize(m.event), "hvdhip_event_synchronize")
         finally:
+            for m in request.markers:
+                m.refs -= 1
+                if m.refs == 0:  # the last request of the response hands the event back to its pool
+                    check(lib().hvdhip_event_release(m.stream.handle, m.event), "hvdhip_event_release")
             request.markers = []
             request.keepalive = []
             for e in request.entries:
