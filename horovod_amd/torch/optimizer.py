@@ -10,7 +10,8 @@ is handed to ``allreduce_async_`` as soon as it has been accumulated
 
 ``synchronize()`` waits for all of them before ``step()`` applies the update.  Parameters
 listed in ``groups`` go out as one grouped request when the last gradient of the group
-arrives (optimizer.py:208-213,236-247).
+arrives (optimizer.py:208-213,236-247).  With ``op=Adasum`` in a world of more than one rank
+the factory returns the delta-based variant (optimizer.py:333-503) instead.
 
 Two things differ from the reference on purpose.  The ROCm refusal of
 ``gradient_predivide_factor`` (optimizer.py:570-572) is gone, because the scale kernels it
@@ -28,30 +29,37 @@ from .compression import Compression
 from .mpi_ops import Adasum, Average
 
 
+def _checked_names(param_groups, named_parameters):
+    """(name, parameter) for every parameter: the caller's list, validated like
+    optimizer.py:41-66, or generated names."""
+    if named_parameters is not None:
+        named_parameters = list(named_parameters)
+    else:
+        named_parameters = [('allreduce.noname.%d.%d' % (i, j), v)
+                            for i, group in enumerate(param_groups)
+                            for j, v in enumerate(group['params'])]
+    if any(not isinstance(p, tuple) for p in named_parameters):
+        raise ValueError('named_parameters should be a sequence of tuples (name, parameter), '
+                         'usually produced by model.named_parameters().')
+    names = [k for k, _ in named_parameters]
+    dups = sorted({k for k in names if names.count(k) > 1})
+    if dups:
+        raise ValueError('Parameter names in named_parameters must be unique. '
+                         'Found duplicates: %s' % ', '.join(dups))
+    all_ids = {id(v) for group in param_groups for v in group['params']}
+    unnamed = all_ids - {id(v) for _, v in named_parameters}
+    if unnamed:
+        raise ValueError('named_parameters was specified, but one or more model parameters were not '
+                         'named. Python object ids: %s' % ', '.join(str(i) for i in unnamed))
+    return named_parameters
+
+
 class _DistributedOptimizer(torch.optim.Optimizer):
     def __init__(self, params, named_parameters, compression, backward_passes_per_step=1, op=Average,
                  gradient_predivide_factor=1.0, groups=None, sparse_as_dense=False):
         super(self.__class__, self).__init__(params)
         self._compression = compression
-        if named_parameters is not None:
-            named_parameters = list(named_parameters)
-        else:
-            named_parameters = [('allreduce.noname.%d.%d' % (i, j), v)
-                                for i, group in enumerate(self.param_groups)
-                                for j, v in enumerate(group['params'])]
-        if any(not isinstance(p, tuple) for p in named_parameters):
-            raise ValueError('named_parameters should be a sequence of tuples (name, parameter), '
-                             'usually produced by model.named_parameters().')
-        names = [k for k, _ in named_parameters]
-        dups = sorted({k for k in names if names.count(k) > 1})
-        if dups:
-            raise ValueError('Parameter names in named_parameters must be unique. '
-                             'Found duplicates: %s' % ', '.join(dups))
-        all_ids = {id(v) for group in self.param_groups for v in group['params']}
-        unnamed = all_ids - {id(v) for _, v in named_parameters}
-        if unnamed:
-            raise ValueError('named_parameters was specified, but one or more model parameters were not '
-                             'named. Python object ids: %s' % ', '.join(str(i) for i in unnamed))
+        named_parameters = _checked_names(self.param_groups, named_parameters)
         self._parameter_names = {v: k for k, v in sorted(named_parameters)}
         self.backward_passes_per_step = backward_passes_per_step
         self._allreduce_delay = {v: backward_passes_per_step for _, v in sorted(named_parameters)}
@@ -243,6 +251,100 @@ class _DistributedOptimizer(torch.optim.Optimizer):
         super(self.__class__, self).load_state_dict(*args, **kwargs)
 
 
+class _DistributedAdasumOptimizer(torch.optim.Optimizer):
+    """Adasum combines parameter *updates*, not gradients (horovod/torch/optimizer.py:333-503).
+
+    When a parameter's gradient is complete the wrapped optimizer steps on that parameter
+    alone; the difference to the value before the step (the delta) replaces the parameter's
+    data and goes out as an in-place ``allreduce_async_(op=Adasum)``.  ``step()`` waits for the
+    combined deltas and sets every parameter to its value before the local step plus the
+    combined delta."""
+
+    def __init__(self, params, named_parameters, compression, backward_passes_per_step=1):
+        super(self.__class__, self).__init__(params)
+        self._compression = compression
+        named_parameters = _checked_names(self.param_groups, named_parameters)
+        self._parameter_names = {v: k for k, v in sorted(named_parameters)}
+        self.backward_passes_per_step = backward_passes_per_step
+        self._allreduce_delay = {v: backward_passes_per_step for _, v in sorted(named_parameters)}
+        self._handles = {}
+        self._hooks = []
+        self._requires_update = set()
+        self._starting_models = {p: torch.zeros_like(p, requires_grad=False) for _, p in named_parameters}
+        for group in self.param_groups:
+            for p in group['params']:
+                if p.requires_grad:
+                    p.grad = p.data.new(p.size()).zero_()
+                    self._requires_update.add(p)
+                    self._hooks.append(p.register_post_accumulate_grad_hook(self._make_hook(p)))
+
+    def set_backward_passes_per_step(self, passes):
+        self.backward_passes_per_step = passes
+        for p in self._allreduce_delay:
+            self._allreduce_delay[p] = passes
+
+    def _allreduce_grad_async(self, p):
+        start = self._starting_models[p]
+        kept = [group['params'] for group in self.param_groups]
+        try:
+            for group in self.param_groups:  # the wrapped optimizer steps on p alone
+                group['params'] = [p] if any(p is v for v in group['params']) else []
+            start.data.copy_(p)
+            super(self.__class__, self).step()
+            p.data.sub_(start)  # p now holds the delta of the local step
+        finally:
+            for group, params in zip(self.param_groups, kept):
+                group['params'] = params
+        compressed, ctx = self._compression.compress(p)
+        handle = mpi_ops.allreduce_async_(compressed.data, name=self._parameter_names.get(p), op=Adasum)
+        return handle, ctx
+
+    def _make_hook(self, p):
+        def hook(*ignore):
+            if p in self._handles and self._handles[p][0] is not None and self._allreduce_delay[p] <= 0:
+                raise AssertionError(
+                    "Gradients were computed more than backward_passes_per_step times before call to step(). "
+                    "Increase backward_passes_per_step to accumulate gradients locally.")
+            assert not p.grad.requires_grad
+            assert self._allreduce_delay[p] > 0
+            handle, ctx = None, None
+            self._allreduce_delay[p] -= 1
+            if self._allreduce_delay[p] == 0:
+                handle, ctx = self._allreduce_grad_async(p)
+            self._handles[p] = (handle, ctx)
+        return hook
+
+    def synchronize(self):
+        pass
+
+    @contextmanager
+    def skip_synchronize(self):
+        raise AssertionError("Skipping synchronization is not supported when using Adasum optimizer.")
+        yield  # pragma: no cover
+
+    def step(self, closure=None):
+        loss = closure() if closure is not None else None
+        for p in self._requires_update - set(self._handles):
+            self._handles[p] = self._allreduce_grad_async(p)
+        for p, (handle, ctx) in list(self._handles.items()):
+            if handle is None:  # step() before the last of backward_passes_per_step passes
+                handle, ctx = self._handles[p] = self._allreduce_grad_async(p)
+            delta = self._compression.decompress(mpi_ops.synchronize(handle), ctx)
+            start = self._starting_models[p]
+            start.data.add_(delta.data)
+            p.data.copy_(start)
+            self._allreduce_delay[p] = self.backward_passes_per_step
+        self._handles.clear()
+        return loss
+
+    def zero_grad(self, *args, **kwargs):
+        if self._handles:
+            raise AssertionError("optimizer.zero_grad() was called after loss.backward() but before "
+                                 "optimizer.step() or optimizer.synchronize(). This is prohibited as it can "
+                                 "cause a race condition.")
+        return super(self.__class__, self).zero_grad(*args, **kwargs)
+
+
 def DistributedOptimizer(optimizer, named_parameters=None, compression=Compression.none,
                          backward_passes_per_step=1, op=Average, gradient_predivide_factor=1.0,
                          num_groups=0, groups=None, sparse_as_dense=False):
@@ -257,9 +359,9 @@ def DistributedOptimizer(optimizer, named_parameters=None, compression=Compressi
                       DeprecationWarning)
         if groups is None:
             groups = num_groups
-    if op == Adasum and mpi_ops.size() > 1:
-        raise NotImplementedError('the delta-based Adasum optimizer (optimizer.py:333-503) is not part of this '
-                                  'build; use hvd.allreduce(op=hvd.Adasum) on the deltas')
-    cls = type(optimizer.__class__.__name__, (optimizer.__class__,), dict(_DistributedOptimizer.__dict__))
-    return cls(optimizer.param_groups, named_parameters, compression, backward_passes_per_step, op,
-               gradient_predivide_factor, groups, sparse_as_dense)
+    if op != Adasum or mpi_ops.size() == 1:
+        cls = type(optimizer.__class__.__name__, (optimizer.__class__,), dict(_DistributedOptimizer.__dict__))
+        return cls(optimizer.param_groups, named_parameters, compression, backward_passes_per_step, op,
+                   gradient_predivide_factor, groups, sparse_as_dense)
+    cls = type(optimizer.__class__.__name__, (optimizer.__class__,), dict(_DistributedAdasumOptimizer.__dict__))
+    return cls(optimizer.param_groups, named_parameters, compression, backward_passes_per_step)

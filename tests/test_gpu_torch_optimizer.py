@@ -140,5 +140,39 @@ def test_argument_checks(hvd):
         hvd.DistributedOptimizer(sgd, named_parameters=[("a", p) for p in model.parameters()])
     with pytest.raises(ValueError, match="not named"):
         hvd.DistributedOptimizer(sgd, named_parameters=list(model.named_parameters())[:1])
-    with pytest.raises(NotImplementedError):
-        hvd.DistributedOptimizer(sgd, op=hvd.Adasum)
+
+
+def test_adasum_optimizer_combines_deltas(hvd, orc):
+    """optimizer.py:333-503: each rank steps locally, the deltas are combined with Adasum and
+    added to the value before the step."""
+    from oracle_util import F32
+    size = 2
+    lr = 0.1
+
+    def peer_delta(rank, name, tensor):
+        g = torch.Generator(device="cuda")
+        g.manual_seed(77 + len(name))
+        return torch.randn(tensor.shape, generator=g, device="cuda") * 0.01
+
+    hvd.init(size=size, peer_source=peer_delta)
+    model = _model()
+    grads = _local_grads(model)
+    before = {n: p.detach().clone() for n, p in model.named_parameters()}
+    opt = hvd.DistributedOptimizer(torch.optim.SGD(model.parameters(), lr=lr),
+                                   named_parameters=model.named_parameters(), op=hvd.Adasum)
+    assert isinstance(opt, torch.optim.SGD) and hasattr(opt, "_starting_models")
+    model.zero_grad()
+    torch.manual_seed(4)
+    model(torch.randn(16, 20, device="cuda")).pow(2).sum().backward()
+    assert len(opt._handles) == 4
+    with pytest.raises(AssertionError, match="not supported"):
+        with opt.skip_synchronize():
+            pass
+    opt.step()
+    for n, p in model.named_parameters():
+        local = (-lr * grads[n]).cpu().numpy().reshape(-1)
+        peer = peer_delta(1, "allreduce." + n, p).cpu().numpy().reshape(-1)
+        combined = orc.adasum_pairwise(local, peer, [local.size], F32)[0]
+        want = before[n].cpu().numpy().reshape(-1) + combined
+        assert np.allclose(p.detach().cpu().numpy().reshape(-1), want, rtol=1e-6, atol=1e-8), n
+    opt.zero_grad()
