@@ -50,9 +50,21 @@ void hvd_adapter_destroy(void* handle) {
   delete h;
 }
 
+int hvd_adapter_allreduce_wire(void* handle, const void* const* tensors, void* const* outputs,
+                               const int64_t* counts, int n, int dtype, int buffer_dtype, double prescale,
+                               double postscale, const void* const* peers, int npeers, char* err, size_t errlen);
+
 int hvd_adapter_allreduce(void* handle, const void* const* tensors, void* const* outputs, const int64_t* counts,
                           int n, int dtype, double prescale, double postscale, const void* const* peers,
                           int npeers, char* err, size_t errlen) {
+  return hvd_adapter_allreduce_wire(handle, tensors, outputs, counts, n, dtype, -1, prescale, postscale, peers,
+                                    npeers, err, errlen);
+}
+
+// buffer_dtype: the dtype of the fusion buffer and of the peers' buffers (-1: that of the tensors).
+int hvd_adapter_allreduce_wire(void* handle, const void* const* tensors, void* const* outputs,
+                               const int64_t* counts, int n, int dtype, int buffer_dtype, double prescale,
+                               double postscale, const void* const* peers, int npeers, char* err, size_t errlen) {
   Harness* h = static_cast<Harness*>(handle);
   try {
     std::vector<TensorTableEntry> entries((size_t)n);
@@ -62,6 +74,7 @@ int hvd_adapter_allreduce(void* handle, const void* const* tensors, void* const*
       entries[(size_t)i].output_data = outputs[i];
       entries[(size_t)i].num_elements = counts[i];
       entries[(size_t)i].dtype = (DataType)dtype;
+      entries[(size_t)i].buffer_dtype = buffer_dtype;
       entries[(size_t)i].device = 0;
     }
     std::vector<const void*> p(peers, peers + npeers);

@@ -174,7 +174,7 @@ gpuStream_t GPUAllreduce::Stream(const std::vector<TensorTableEntry>& entries) {
 hvdhip_fusion_plan* GPUAllreduce::PlanFor(const std::vector<TensorTableEntry>& entries) {
   std::vector<uint64_t> key;
   key.reserve(3 * entries.size() + 1);
-  key.push_back((uint64_t)entries[0].dtype);
+  key.push_back((uint64_t)entries[0].dtype | ((uint64_t)entries[0].wire_dtype() << 8));
   for (auto& e : entries) {
     key.push_back((uint64_t)(uintptr_t)e.tensor_data);
     key.push_back((uint64_t)(uintptr_t)e.output_data);
@@ -204,7 +204,7 @@ hvdhip_fusion_plan* GPUAllreduce::PlanFor(const std::vector<TensorTableEntry>& e
   hvdhip_fusion_plan* plan = nullptr;
   gpu_context_->ErrorCheck("hvdhip_fusion_plan_create",
                            hvdhip_fusion_plan_create(tensors.data(), outputs.data(), counts.data(), (int)entries.size(),
-                                                     (int)entries[0].dtype, (int)entries[0].dtype, &plan));
+                                                     (int)entries[0].dtype, (int)entries[0].wire_dtype(), &plan));
   plans_[key] = plan;
   plan_order_.push_front(key);
   return plan;
@@ -219,9 +219,14 @@ void GPUAllreduce::ScaleMemcpyInFusionBuffer(const std::vector<TensorTableEntry>
                                              const void*& fused_input_data, void*& buffer_data,
                                              size_t& buffer_len, double scale_factor) {
   buffer_data = global_state_->fusion_buffer[(size_t)global_state_->current_nccl_stream];
+  const bool converting = entries[0].wire_dtype() != entries[0].dtype;
+  if (converting && !global_state_->batch_d2d_memcopies)
+    throw std::logic_error("A fusion buffer of another dtype than the tensors needs HOROVOD_BATCH_D2D_MEMCOPIES.");
   if (global_state_->batch_d2d_memcopies) {
     hvdhip_fusion_plan* plan = PlanFor(entries);
-    int rc = hvdhip_fusion_pack(plan, buffer_data, scale_factor, HVDHIP_PACK_DEFAULT, Stream(entries));
+    // cast, then scale the half: the order (and roundings) of compress() followed by the fp16 ScaleBuffer
+    int rc = hvdhip_fusion_pack(plan, buffer_data, scale_factor,
+                                converting ? HVDHIP_PACK_CAST_THEN_SCALE : HVDHIP_PACK_DEFAULT, Stream(entries));
     if (rc == HVDHIP_ERR_UNSUPPORTED_DTYPE)  // ops/cuda/cuda_kernels.cu:317-319
       throw std::logic_error("Type " + DataType_Name(entries[0].dtype) +
                              " not supported by BatchedScaledD2DMemcpyCudaImpl.");
@@ -292,7 +297,9 @@ void GPUAllreduce::Execute(std::vector<TensorTableEntry>& entries, double presca
   void* buffer_data;
   size_t buffer_len;
   const bool timeline = global_state_->timeline_initialized;
-  if (entries.size() > 1) {
+  const DataType wire = first_entry.wire_dtype();
+  const bool fused = entries.size() > 1 || wire != first_entry.dtype;  // a lone entry still needs the buffer to convert
+  if (fused) {
     ScaleMemcpyInFusionBuffer(entries, fused_input_data, buffer_data, buffer_len, prescale_factor);
     if (timeline) gpu_context_->RecordEvent(gpu_op_context_.event_queue, MEMCPY_IN_FUSION_BUFFER, *gpu_op_context_.stream);
   } else {
@@ -310,18 +317,18 @@ void GPUAllreduce::Execute(std::vector<TensorTableEntry>& entries, double presca
   }
   // The collective (ncclAllReduce(sum), ops/nccl_operations.cc:190-193) on one GPU.
   if (!peers.empty()) {
-    int64_t num_elements = (int64_t)(buffer_len / DataType_Size(first_entry.dtype));
+    int64_t num_elements = (int64_t)(buffer_len / DataType_Size(wire));
     size_t done = 0;
     while (done < peers.size()) {
       int k = (int)std::min<size_t>(16, peers.size() - done);
       gpu_context_->ErrorCheck("hvdhip_reduce_sum_k",
-                               hvdhip_reduce_sum_k(buffer_data, peers.data() + done, k, num_elements,
-                                                   (int)first_entry.dtype, Stream(entries)));
+                               hvdhip_reduce_sum_k(buffer_data, peers.data() + done, k, num_elements, (int)wire,
+                                                   Stream(entries)));
       done += (size_t)k;
     }
   }
   if (timeline) gpu_context_->RecordEvent(gpu_op_context_.event_queue, NCCL_ALLREDUCE, *gpu_op_context_.stream);
-  if (entries.size() > 1) {
+  if (fused) {
     ScaleMemcpyOutFusionBuffer(buffer_data, buffer_len, postscale_factor, entries);
     if (timeline) gpu_context_->RecordEvent(gpu_op_context_.event_queue, MEMCPY_OUT_FUSION_BUFFER, *gpu_op_context_.stream);
   } else if (postscale_factor != 1.0) {

@@ -62,6 +62,11 @@ struct TensorTableEntry {
   DataType dtype = HOROVOD_FLOAT32;
   int device = 0;
   int64_t tensor_size() const { return num_elements * (int64_t)DataType_Size(dtype); }
+  // Not in the reference: the dtype the entry travels in.  HOROVOD_FLOAT16 with FLOAT32 tensors
+  // folds Compression.fp16 (horovod/torch/compression.py:46-64) into packing and unpacking;
+  // left at its default the entry travels as it is.
+  int buffer_dtype = -1;
+  DataType wire_dtype() const { return buffer_dtype < 0 ? dtype : (DataType)buffer_dtype; }
 };
 
 // common/common.h:181-189

@@ -20,7 +20,7 @@ def test_adapter_loads_and_exports_its_test_surface():
     lib = _load()
     for name in ("hvd_adapter_create", "hvd_adapter_destroy", "hvd_adapter_allreduce", "hvd_adapter_state",
                  "hvd_adapter_adasum_pairwise", "hvd_adapter_adasum_dispatch", "hvd_adapter_fuse",
-                 "hvd_adapter_fuse_keyed"):
+                 "hvd_adapter_fuse_keyed", "hvd_adapter_allreduce_wire"):
         assert hasattr(lib, name)
 
 

@@ -25,6 +25,10 @@ def adapter(gpu):
     lib.hvd_adapter_allreduce.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                           ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_double,
                                           ctypes.c_void_p, ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t]
+    lib.hvd_adapter_allreduce_wire.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                               ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_double,
+                                               ctypes.c_double, ctypes.c_void_p, ctypes.c_int, ctypes.c_char_p,
+                                               ctypes.c_size_t]
     lib.hvd_adapter_state.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
     lib.hvd_adapter_adasum_pairwise.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                                 ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_char_p,
@@ -54,6 +58,13 @@ class Harness:
         cnt = (ctypes.c_int64 * len(counts))(*counts)
         rc = self.lib.hvd_adapter_allreduce(self.h, _ptrs(tensors), _ptrs(outputs), cnt, len(counts), dtype,
                                             prescale, postscale, _ptrs(list(peers)), len(peers), err, 512)
+        return rc, err.value.decode()
+
+    def allreduce_wire(self, tensors, outputs, counts, dtype, wire, prescale, postscale, peers=()):
+        err = ctypes.create_string_buffer(512)
+        cnt = (ctypes.c_int64 * len(counts))(*counts)
+        rc = self.lib.hvd_adapter_allreduce_wire(self.h, _ptrs(tensors), _ptrs(outputs), cnt, len(counts), dtype, wire,
+                                                 prescale, postscale, _ptrs(list(peers)), len(peers), err, 512)
         return rc, err.value.decode()
 
     def state(self):
@@ -111,6 +122,52 @@ def test_execute_fused_matches_the_cpu_op_sequence(gpu, orc, adapter, batch, dty
         cur, plans = h.state()
         assert cur == 3 % 2  # current_nccl_stream rotated after every op (ops/gpu_operations.cc:101-103)
         assert plans == (1 if batch else 0)
+    finally:
+        h.close()
+
+
+@pytest.mark.parametrize("counts", [[5, 1000, 3, 70001, 256, 1], [4099]])
+def test_execute_with_an_fp16_fusion_buffer_folds_the_compression_cast(gpu, orc, adapter, counts):
+    """float32 entries, float16 fusion buffer and peers: cast (RNE), fp16 prescale, fp16 sums in
+    peer order, fp16 postscale, exact widening: what Compression.fp16 around an fp16 allreduce
+    computes (horovod/torch/compression.py:46-64), with no half tensors.  A lone entry goes
+    through the buffer too, because the conversion needs somewhere to land."""
+    rng = np.random.default_rng(5)
+    src, dst = Arena(1 << 20), Arena(1 << 20, fill=0x5A)
+    so, do, vals = [], [], []
+    for c in counts:
+        so.append(src.alloc(c * 4)), do.append(dst.alloc(c * 4))
+        v = (rng.standard_normal(c) * 1e-3).astype(np.float32)
+        src.host[so[-1]:so[-1] + c * 4] = v.view(np.uint8)
+        vals.append(v)
+    src.upload(), dst.upload()
+    offs = orc.padded_offsets([c * 2 for c in counts])
+    peer_vals = [[(rng.standard_normal(c) * 1e-3).astype(np.float16) for c in counts] for _ in range(3)]
+    peers = []
+    for pv in peer_vals:
+        img = np.zeros(int(offs[-1]) + 64, np.uint8)
+        for o, v in zip(offs, pv):
+            img[o:o + v.nbytes] = v.view(np.uint8)
+        peers.append(gpu.upload(img))
+    h = Harness(adapter, gpu, num_streams=1)
+    try:
+        rc, msg = h.allreduce_wire([src.ptr(o) for o in so], [dst.ptr(o) for o in do], counts, F32, F16, 0.125, 0.5,
+                                   [p.data_ptr() for p in peers])
+        assert rc == 0, msg
+        out = dst.download()
+        for i, (c, v) in enumerate(zip(counts, vals)):
+            w = orc.scale_cast_f32_to_f16(v, 0.125, cast_first=True)
+            for pv in peer_vals:
+                w = orc.float16_sum(pv[i].view(np.uint16), w)
+            want = orc.scale_cast_f16_to_f32(w, 0.5)
+            assert np.array_equal(out[do[i]:do[i] + c * 4], want.view(np.uint8)), "entry %d" % i
+        assert h.state()[1] == 1
+    finally:
+        h.close()
+    h = Harness(adapter, gpu, num_streams=1, batch=False)
+    try:
+        rc, msg = h.allreduce_wire([src.ptr(o) for o in so], [dst.ptr(o) for o in do], counts, F32, F16, 1.0, 1.0)
+        assert rc != 0 and "HOROVOD_BATCH_D2D_MEMCOPIES" in msg
     finally:
         h.close()
 
