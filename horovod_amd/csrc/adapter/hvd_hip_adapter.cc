@@ -435,7 +435,8 @@ void AdasumGPU::FusedPairwiseReduce(void* a, const void* b, DataType horovod_dat
                                     const std::vector<int>& tensor_counts, std::vector<double>* normAndDots,
                                     gpuStream_t stream) {
   CheckAdasumType(horovod_datatype, "FusedPairwiseReduce");
-  auto key = std::make_pair((int)horovod_datatype, tensor_counts);
+  // a plan owns the partial sums of the combine in flight, so streams do not share one
+  auto key = std::make_pair(std::make_pair((int)horovod_datatype, (const void*)stream), tensor_counts);
   hvdhip_adasum_plan* plan;
   auto it = plans_.find(key);
   if (it == plans_.end()) {

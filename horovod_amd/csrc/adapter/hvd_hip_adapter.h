@@ -225,7 +225,7 @@ public:
 
 private:
   GPUContext* gpu_context_;
-  std::map<std::pair<int, std::vector<int>>, hvdhip_adasum_plan*> plans_;
+  std::map<std::pair<std::pair<int, const void*>, std::vector<int>>, hvdhip_adasum_plan*> plans_;  // (dtype, stream), counts
 };
 
 // Controller::FuseResponses (common/controller.cc:793-866) for allreduce responses of one

@@ -166,8 +166,9 @@ class Engine:
         self.plans[key] = plan
         return plan
 
-    def _adasum_plan(self, layer_counts, dtype):
-        key = (tuple(layer_counts), dtype)
+    def _adasum_plan(self, slot, layer_counts, dtype):
+        # an Adasum plan owns the partial sums of the combine in flight: one per stream slot
+        key = (slot, tuple(layer_counts), dtype)
         plan = self.adasum_plans.get(key)
         if plan is None:
             if len(self.adasum_plans) >= self.max_plans:
@@ -243,7 +244,7 @@ class Engine:
 
         if nelem and peer_bufs:
             if first.op == ADASUM:
-                self._adasum(result, peer_bufs, nelem, layer_counts, wire, s)
+                self._adasum(slot, result, peer_bufs, nelem, layer_counts, wire, s)
             else:
                 self._sum(result, peer_bufs, nelem, wire, s)
 
@@ -275,7 +276,7 @@ class Engine:
         for i in range(0, len(peer_bufs), 16):
             H.reduce_sum_k(result, peer_bufs[i:i + 16], nelem, dtype, s)
 
-    def _adasum(self, result, peer_bufs, nelem, layer_counts, dtype, s):
+    def _adasum(self, slot, result, peer_bufs, nelem, layer_counts, dtype, s):
         """Ranks of one node are summed (the reduce-scatter leg of
         ops/adasum_gpu_operations.cc:174-197), then the node results are combined pairwise at
         distances 1, 2, 4 ... like the levels of Adasum::FusedAllreduce (ops/adasum/adasum.h:194-340)."""
@@ -287,7 +288,7 @@ class Engine:
             if L > 1:
                 self._sum(lead, bufs[node * L + 1:node * L + L], nelem, dtype, s)
             leaders.append(lead)
-        plan = self._adasum_plan(layer_counts, dtype)
+        plan = self._adasum_plan(slot, layer_counts, dtype)
         d = 1
         while d < len(leaders):
             for i in range(0, len(leaders), 2 * d):

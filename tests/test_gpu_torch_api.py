@@ -375,3 +375,21 @@ def test_fuzz_against_the_oracle(hvd, orc, seed):
         assert out.numel() == n
         if n:
             assert np.array_equal(_np(out).reshape(-1).view(np.uint8), np.ascontiguousarray(want).view(np.uint8)), name
+
+
+def test_adasum_responses_on_alternating_streams_do_not_share_state(hvd, orc):
+    """Equal-shaped Adasum responses of one cycle run on different streams at the same time;
+    each stream slot keeps Adasum partial sums of its own."""
+    hvd.init(size=2, peer_source=_peer_values, fusion_threshold=1 << 20, num_streams=2)
+    torch.manual_seed(21)
+    tensors = [torch.randn(200000, device="cuda") for _ in range(6)]  # 800 KB each: one response per tensor
+    names = ["t%d" % i for i in range(6)]
+    handles = [hvd.allreduce_async(t, name=n, op=hvd.Adasum) for t, n in zip(tensors, names)]
+    outs = [hvd.synchronize(h) for h in handles]
+    import horovod_amd.torch.mpi_ops as ops
+    assert ops._engine.responses == 6
+    for t, n, out in zip(tensors, names, outs):
+        peer = _np(_peer_values(1, "allreduce." + n, t))
+        want = orc.adasum_pairwise(_np(t), peer, [t.numel()], F32)[0]
+        ulp = np.abs(_np(out).view(np.int32).astype(np.int64) - want.view(np.int32).astype(np.int64))
+        assert ulp.max() <= 1, n
