@@ -318,10 +318,11 @@ def extras(steps, warmup):
         es = 4 if tdtype == DTYPE["float32"] else 2
         counts = [W.numel(s) for s in shapes]
         reps = []
+        shared = [Stream() for _ in range(streams)]  # every replica queues on the same stream(s)
         for r in range(replicas):
             src = DeviceSet(counts, es, lambda n: randn(n, tt[tdtype], std, 1 + r))
             dst = DeviceSet(counts, es, lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
-            pipe = AllreducePipeline(src.ptrs, dst.ptrs, counts, tdtype, bdtype, num_streams=streams)
+            pipe = AllreducePipeline(src.ptrs, dst.ptrs, counts, tdtype, bdtype, streams=shared)
             bs = 4 if pipe.buffer_dtype == DTYPE["float32"] else 2
             max_elems = max(c.buffer_elems for c in pipe.cycles)
             peer_bufs = []
@@ -351,12 +352,15 @@ def extras(steps, warmup):
                      "replicas_rotated": replicas}
         for _, _, pipe, _ in reps:
             pipe.destroy()
+        for st in shared:
+            st.destroy()
         del reps
         torch.cuda.empty_cache()
 
     F32, F16 = DTYPE["float32"], DTYPE["float16"]
     run_pipeline("resnet50_fp32_pack_scale_reduce_unpack", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0, 1,
                  replicas=4)
+    run_pipeline("resnet50_fp32_two_streams", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0, 2, replicas=4)
     run_pipeline("bert_large_fp32_to_fp16_7peers_eighth_chunk", W.bert_large_shapes(), F32, F16, 1e-4, 7, 0.125, 1,
                  steps_=max(5, steps // 10))
     run_pipeline("gpt2_xl_fp16_two_streams", W.gpt2_xl_shapes(), F16, F16, 1e-3, 1, 1.0, 2,
@@ -495,7 +499,7 @@ def main():
         # stream slot as in common/fusion_buffer_manager.cc): the start-up and drain of one step's kernels
         # overlap the other's.  Reported beside the headline value, which stays single-stream.
         try:
-            pair = [stream, Stream()]
+            pair = [Stream(), Stream()]
 
             def step2():
                 i = turn[0] = (turn[0] + 1) % len(plans)
@@ -510,6 +514,7 @@ def main():
             two_streams = {"GB/s": round(4 * payload / sec2 / 1e9, 1),
                            "frac_of_hbm_peak": round(4 * payload / sec2 / 1e9 / HBM_PEAK_GBS, 4),
                            "ms_per_step": round(sec2 * 1e3, 5), "streams": 2}
+            pair[0].destroy()
             pair[1].destroy()
         except Exception as e:  # pragma: no cover
             two_streams = {"error": "%s: %s" % (type(e).__name__, e)}

@@ -43,11 +43,14 @@ class AllreducePipeline:
     share)."""
 
     def __init__(self, tensor_ptrs, output_ptrs, counts, tensor_dtype, buffer_dtype=None,
-                 threshold=FUSION_THRESHOLD, num_streams=1, completion_events=None):
+                 threshold=FUSION_THRESHOLD, num_streams=1, completion_events=None, streams=None):
         """completion_events: record a pooled event after every cycle and wait on those in
         synchronize(), as GPUOpContext::FinalizeGPUQueue does (about 2 us of stream time per
         event).  Default: on when cycles alternate over several streams, off for one stream,
-        where synchronize() simply waits for the stream."""
+        where synchronize() simply waits for the stream.
+
+        streams: existing Stream objects to run on instead of creating num_streams new ones
+        (they stay with the caller), so that several pipelines queue on the same streams."""
         self.tensor_dtype = int(tensor_dtype)
         self.buffer_dtype = int(tensor_dtype if buffer_dtype is None else buffer_dtype)
         ts, bs = dtype_size(self.tensor_dtype), dtype_size(self.buffer_dtype)
@@ -69,7 +72,9 @@ class AllreducePipeline:
             n = sum(counts[i] for i in g)
             cyc.payload_in, cyc.payload_buf, cyc.payload_out = n * ts, n * bs, n * ts
             self.cycles.append(cyc)
-        self.streams = [H.Stream() for _ in range(num_streams)]
+        self.owns_streams = streams is None
+        self.streams = [H.Stream() for _ in range(num_streams)] if streams is None else list(streams)
+        num_streams = len(self.streams)
         self.completion_events = (num_streams > 1) if completion_events is None else bool(completion_events)
         self.pending = []  # (stream, event) recorded after each cycle
         self.buffers = [torch.empty(max(max_len, 16), dtype=torch.uint8, device="cuda") for _ in range(num_streams)]
@@ -143,5 +148,6 @@ class AllreducePipeline:
         for cyc in self.cycles:
             if cyc.plan is not None:
                 cyc.plan.destroy()
-        for s in self.streams:
-            s.destroy()
+        if self.owns_streams:
+            for s in self.streams:
+                s.destroy()
