@@ -66,3 +66,18 @@ def test_missing_library_fails_loudly(monkeypatch):
         assert "no fallback" in str(e)
     else:
         raise AssertionError("loading a missing library must raise")
+
+
+def test_header_is_plain_c99():
+    """The boundary is a C ABI: the header must compile as C, warnings as errors."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", "c",
+                        os.path.join(root, "include", "hvdhip.h")], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+
+
+def test_c_client_is_built_with_the_library():
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    assert os.path.exists(os.path.join(root, "horovod_amd", "lib", "c_client")), \
+        "make -C horovod_amd/csrc builds the C99 example next to the library"
