@@ -50,6 +50,10 @@ def parse():
                          "Adasum combine of 2 x 2^25 fp32 in 64 layers")
     ap.add_argument("--calibrate", action="store_true",
                     help="only launch a plain 256 MiB device copy (scales rocprofv3 byte counters)")
+    ap.add_argument("--streams", type=int, default=2,
+                    help="stream slots the headline steps alternate over, each with a fusion buffer of its own "
+                         "(HOROVOD_NUM_NCCL_STREAMS); default 2, the configuration this library is meant to run "
+                         "in; the one-stream figure is reported beside it")
     ap.add_argument("--replicas", type=int, default=8,
                     help="independent copies of the workload that steps rotate over, so that the "
                          "bytes touched between two uses of one copy exceed the 256 MB Infinity Cache")
@@ -299,6 +303,19 @@ def per_tensor_comparator(counts, src, dst, reps=20):
     return out
 
 
+_PAIR = []
+
+
+def stream_pair():
+    """Two library streams created once, before any other, and shared by everything in this run
+    that alternates over stream slots: streams that are created later, while others exist, can
+    land on a hardware queue that is already in use and then overlap nothing."""
+    if not _PAIR:
+        from horovod_amd import Stream
+        _PAIR.extend([Stream(), Stream()])
+    return _PAIR
+
+
 def extras(steps, warmup):
     """The other pipelines, each as algorithmic GB/s and fraction of the HBM peak."""
     import torch
@@ -318,7 +335,7 @@ def extras(steps, warmup):
         es = 4 if tdtype == DTYPE["float32"] else 2
         counts = [W.numel(s) for s in shapes]
         reps = []
-        shared = [Stream() for _ in range(streams)]  # every replica queues on the same stream(s)
+        shared = stream_pair()[:streams]  # every replica queues on the same stream(s)
         for r in range(replicas):
             src = DeviceSet(counts, es, lambda n: randn(n, tt[tdtype], std, 1 + r))
             dst = DeviceSet(counts, es, lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
@@ -352,8 +369,6 @@ def extras(steps, warmup):
                      "replicas_rotated": replicas}
         for _, _, pipe, _ in reps:
             pipe.destroy()
-        for st in shared:
-            st.destroy()
         del reps
         torch.cuda.empty_cache()
 
@@ -378,7 +393,7 @@ def extras(steps, warmup):
         b = 0.3 * a + (1 - 0.09) ** 0.5 * torch.randn(n, generator=g, device="cuda", dtype=torch.float32)
         pairs.append((a, b))
     plan = AdasumPlan(counts, F32)
-    s = Stream()
+    s = stream_pair()[0]
     torch.cuda.synchronize()
     turn = [0]
 
@@ -394,7 +409,6 @@ def extras(steps, warmup):
                                          "ms": round(sec * 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1),
                                          "replicas_rotated": len(pairs)}
     plan.destroy()
-    s.destroy()
     del pairs
     return out
 
@@ -415,7 +429,7 @@ def main():
     native.ensure_built()  # loads what is built; builds only if nothing is
     horovod_amd.lib()  # fails loudly if the HIP library cannot be loaded
 
-    stream = Stream()
+    stream = stream_pair()[0]
     F32 = DTYPE["float32"]
     if args.calibrate:
         from horovod_amd import host as H
@@ -458,10 +472,19 @@ def main():
         i = turn[0] = (turn[0] + 1) % len(plans)
         plans[i].pack(fbs[i].data_ptr(), 0.125, stream)
 
+    if args.streams not in (1, 2):
+        print("bench.py alternates over one or two stream slots", file=sys.stderr)
+        sys.exit(2)
+    slots = stream_pair()[:args.streams]
+
     def step():
         i = turn[0] = (turn[0] + 1) % len(plans)
-        plans[i].pack(fbs[i].data_ptr(), 0.125, stream)
-        plans[i].unpack(fbs[i].data_ptr(), 1.0, stream)
+        plans[i].pack(fbs[i].data_ptr(), 0.125, slots[i % len(slots)])
+        plans[i].unpack(fbs[i].data_ptr(), 1.0, slots[i % len(slots)])
+
+    def sync_slots():
+        for st in slots:
+            st.synchronize()
 
     if args.kernel_only:
         for _ in range(args.warmup + args.steps):
@@ -469,7 +492,7 @@ def main():
         stream.synchronize()
         return
 
-    sec = timed(step, stream.synchronize, args.steps, args.warmup)
+    sec = timed(step, sync_slots, args.steps, args.warmup)
     value = 4 * payload / sec / 1e9
 
     ksec = event_timed(pack, stream, args.steps, args.warmup)
@@ -485,39 +508,39 @@ def main():
         "ms_per_step": round(sec * 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "fusion stress: 1,024 fp32 tensors, log-uniform 256..65,536 elements (seed 3), "
-                               "U(-1,1) (seed 4); pack with prescale 0.125 into a 64 MiB fusion buffer, unpack",
+                               "U(-1,1) (seed 4); pack with prescale 0.125 into a 64 MiB fusion buffer, unpack; "
+                               "consecutive steps alternate over the stream slots, each slot with its own buffers",
                    "tensors": len(counts), "payload_bytes": payload, "buffer_len": plan.buffer_len,
-                   "algorithmic_bytes_per_step": 4 * payload, "replicas_rotated": len(plans)},
+                   "algorithmic_bytes_per_step": 4 * payload, "replicas_rotated": len(plans),
+                   "streams": len(slots)},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "roofline": roofline,
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline_stress(counts, host)
-    two_streams = None
+    other = None
     if not args.no_extra:
-        # The same steps alternating over two streams (HOROVOD_NUM_NCCL_STREAMS=2, one fusion buffer per
-        # stream slot as in common/fusion_buffer_manager.cc): the start-up and drain of one step's kernels
-        # overlap the other's.  Reported beside the headline value, which stays single-stream.
+        # The same steps with the other stream count: all on one stream when the headline alternates over
+        # several (every kernel then waits for its predecessor, the reference's default
+        # HOROVOD_NUM_NCCL_STREAMS=1), or on two streams when the headline was asked to use one.
         try:
-            pair = [Stream(), Stream()]
+            alt = stream_pair()[:1 if len(slots) > 1 else 2]
 
-            def step2():
+            def step_alt():
                 i = turn[0] = (turn[0] + 1) % len(plans)
-                plans[i].pack(fbs[i].data_ptr(), 0.125, pair[i % 2])
-                plans[i].unpack(fbs[i].data_ptr(), 1.0, pair[i % 2])
+                plans[i].pack(fbs[i].data_ptr(), 0.125, alt[i % len(alt)])
+                plans[i].unpack(fbs[i].data_ptr(), 1.0, alt[i % len(alt)])
 
-            def sync2():
-                pair[0].synchronize()
-                pair[1].synchronize()
+            def sync_alt():
+                for st in alt:
+                    st.synchronize()
 
-            sec2 = timed(step2, sync2, args.steps, args.warmup)
-            two_streams = {"GB/s": round(4 * payload / sec2 / 1e9, 1),
-                           "frac_of_hbm_peak": round(4 * payload / sec2 / 1e9 / HBM_PEAK_GBS, 4),
-                           "ms_per_step": round(sec2 * 1e3, 5), "streams": 2}
-            pair[0].destroy()
-            pair[1].destroy()
+            sec2 = timed(step_alt, sync_alt, args.steps, args.warmup)
+            other = {"GB/s": round(4 * payload / sec2 / 1e9, 1),
+                     "frac_of_hbm_peak": round(4 * payload / sec2 / 1e9 / HBM_PEAK_GBS, 4),
+                     "ms_per_step": round(sec2 * 1e3, 5), "streams": len(alt)}
         except Exception as e:  # pragma: no cover
-            two_streams = {"error": "%s: %s" % (type(e).__name__, e)}
+            other = {"error": "%s: %s" % (type(e).__name__, e)}
     comparator = None
     if not args.no_extra:
         try:
@@ -535,7 +558,7 @@ def main():
         except Exception as e:  # pragma: no cover
             result["extra"] = {"error": "%s: %s" % (type(e).__name__, e)}
         result["extra"]["fusion_stress_execute_vs_per_tensor_copies"] = comparator
-        result["extra"]["fusion_stress_two_streams"] = two_streams
+        result["extra"]["fusion_stress_one_stream" if len(slots) > 1 else "fusion_stress_two_streams"] = other
         if not args.no_cpu and "error" not in result["extra"]:
             try:
                 for name, v in cpu_extras().items():

@@ -44,10 +44,7 @@ void hvd_adapter_destroy(void* handle) {
   if (!h) return;
   delete h->allreduce;
   delete h->adasum;
-  for (auto& m : h->context.streams)
-    for (auto& kv : m)
-      if (kv.second) hvdhip_stream_destroy(kv.second);
-  delete h;
+  delete h;  // the context's destructor gives its streams back
 }
 
 int hvd_adapter_allreduce_wire(void* handle, const void* const* tensors, void* const* outputs,

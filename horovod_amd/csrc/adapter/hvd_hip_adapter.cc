@@ -23,7 +23,13 @@ const std::string& DataType_Name(DataType value) {
 // ---------------------------------------------------------------- GPUContext
 
 GPUContext::GPUContext() {}
-GPUContext::~GPUContext() {}
+// The reference keeps its streams for the life of the process; a context that can be created
+// and dropped many times (tests, benchmarks) gives them back.
+GPUContext::~GPUContext() {
+  for (auto& per_device : streams)
+    for (auto& kv : per_device)
+      if (kv.second) hvdhip_stream_destroy(kv.second);
+}
 
 void GPUContext::ErrorCheck(std::string op_name, int gpu_result) {
   if (gpu_result != 0) {
