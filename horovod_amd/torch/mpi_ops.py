@@ -41,8 +41,9 @@ def init(size=1, local_size=1, peer_source=None, fusion_threshold=None, num_stre
 
     peer_source(rank, name, tensor) returns what rank 1..size-1 passes under that name; None
     means every rank holds the same values.  fusion_threshold and num_streams default to
-    HOROVOD_FUSION_THRESHOLD (bytes, 64 MiB) and HOROVOD_NUM_NCCL_STREAMS (1), the knobs of
-    common/operations.cc:419-441,475-481."""
+    HOROVOD_FUSION_THRESHOLD (bytes, 64 MiB) and HOROVOD_NUM_NCCL_STREAMS, the knobs of
+    common/operations.cc:419-441,475-481; without the variable there are two stream slots (the
+    reference has one): consecutive fused responses then overlap each other's start-up and drain."""
     global _engine
     if _engine is not None:
         return
@@ -52,7 +53,7 @@ def init(size=1, local_size=1, peer_source=None, fusion_threshold=None, num_stre
     if fusion_threshold is None:
         fusion_threshold = int(os.environ.get("HOROVOD_FUSION_THRESHOLD", 64 << 20))
     if num_streams is None:
-        num_streams = int(os.environ.get("HOROVOD_NUM_NCCL_STREAMS", 1))
+        num_streams = int(os.environ.get("HOROVOD_NUM_NCCL_STREAMS", 2))
     batch = os.environ.get("HOROVOD_BATCH_D2D_MEMCOPIES", "1") != "0"
     _engine = Engine(size, local_size, peer_source, fusion_threshold, num_streams, batch)
 
