@@ -378,6 +378,8 @@ def extras(steps, warmup):
     run_pipeline("resnet50_fp32_two_streams", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0, 2, replicas=4)
     run_pipeline("bert_large_fp32_to_fp16_7peers_eighth_chunk", W.bert_large_shapes(), F32, F16, 1e-4, 7, 0.125, 1,
                  steps_=max(5, steps // 10))
+    run_pipeline("bert_large_fp32_to_fp16_two_streams", W.bert_large_shapes(), F32, F16, 1e-4, 7, 0.125, 2,
+                 steps_=max(5, steps // 10))
     run_pipeline("gpt2_xl_fp16_two_streams", W.gpt2_xl_shapes(), F16, F16, 1e-3, 1, 1.0, 2,
                  steps_=max(3, steps // 40))
 
