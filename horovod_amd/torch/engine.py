@@ -43,14 +43,17 @@ class HorovodInternalError(RuntimeError):
 
 
 class Entry:
-    __slots__ = ("name", "tensor", "output", "count")
+    __slots__ = ("name", "tensor", "output", "count", "parts")
 
     def __init__(self, name, tensor, output):
         self.name, self.tensor, self.output, self.count = name, tensor, output, tensor.numel()
+        self.parts = None  # allgather: what every rank contributes, rank 0 first
 
 
 class Request:
-    def __init__(self, entries, op, prescale, postscale, divisor, tensor_dtype, wire_dtype, device):
+    def __init__(self, entries, op, prescale, postscale, divisor, tensor_dtype, wire_dtype, device,
+                 kind="allreduce"):
+        self.kind = kind
         self.entries = entries
         self.op, self.prescale, self.postscale, self.divisor = op, float(prescale), float(postscale), divisor
         self.tensor_dtype, self.wire_dtype, self.device = tensor_dtype, wire_dtype, device
@@ -61,7 +64,7 @@ class Request:
         self.error = None
 
     def key(self):
-        return (self.op, self.device, self.tensor_dtype, self.wire_dtype, self.prescale, self.postscale)
+        return (self.kind, self.op, self.device, self.tensor_dtype, self.wire_dtype, self.prescale, self.postscale)
 
 
 class Marker:
@@ -109,8 +112,33 @@ class Engine:
         # (RecordReadyEvent, horovod/torch/ready_event.cc).  A cycle here runs on the caller's own
         # thread, after every enqueue it serves, so one event per producing stream and cycle, recorded
         # when the cycle starts, orders the same work and costs one record instead of one per tensor.
+        if request.kind == "allgather":
+            self._prepare_allgather(request)
         request.producer = torch.cuda.current_stream()
         self.queue.append(request)
+
+    def _prepare_allgather(self, request):
+        """Collects what every rank passes (first dimensions may differ, the rest may not:
+        AllgatherOp::AllocateOutput, ops/collective_operations.cc:150-198) and allocates the
+        output, here, before the cycle's ready event, so that its memory is ordered like any
+        other tensor of the framework."""
+        for e in request.entries:
+            if e.tensor.dim() == 0:
+                self.inflight.pop(e.name, None)
+                # common/controller.cc:575-579
+                raise HorovodInternalError("Rank zero tried to allgather a rank-zero tensor.")
+            parts = [e.tensor]
+            for rank in range(1, self.size):
+                t = e.tensor if self.peer_source is None else self.peer_source(rank, e.name, e.tensor)
+                if (not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != e.tensor.dtype
+                        or t.dim() != e.tensor.dim() or t.shape[1:] != e.tensor.shape[1:] or not t.is_contiguous()):
+                    self.inflight.pop(e.name, None)
+                    raise HorovodInternalError(
+                        "Mismatched allgather tensor shapes: ranks may differ in the first dimension only "
+                        "(tensor %r)." % e.name)
+                parts.append(t)
+            e.parts = parts
+            e.output.resize_((sum(t.shape[0] for t in parts),) + tuple(e.tensor.shape[1:]))
 
     def run_cycle(self):
         """Fuses and queues everything enqueued so far (one pass of RunLoopOnce,
@@ -127,18 +155,23 @@ class Engine:
                 self.ready[r.producer] = ev
         flat = [(r, e) for r in pending for e in r.entries]
         n = len(flat)
-        sizes = (c_int64 * n)(*[e.count * dtype_size(r.wire_dtype) for r, e in flat])
+        pad = (lambda b: 16 * ((b + 15) // 16)) if self.batch_d2d_memcopies else (lambda b: b)
+        sizes = (c_int64 * n)(*[
+            e.output.numel() * dtype_size(r.tensor_dtype) if r.kind == "allgather"  # no padding on that path
+            else pad(e.count * dtype_size(r.wire_dtype)) for r, e in flat])
         classes = {}
         keys = (c_int * n)(*[classes.setdefault(r.key(), len(classes)) for r, _ in flat])
         group_of = (c_int * n)()
-        ngroups = adapter_lib().hvd_adapter_fuse_keyed(sizes, keys, n, self.fusion_threshold,
-                                                       int(self.batch_d2d_memcopies), group_of)
+        ngroups = adapter_lib().hvd_adapter_fuse_keyed(sizes, keys, n, self.fusion_threshold, 0, group_of)
         groups = [[] for _ in range(ngroups)]
         for i in range(n):
             groups[group_of[i]].append(flat[i])
         for g in groups:
             try:
-                self._execute(g)
+                if g[0][0].kind == "allgather":
+                    self._execute_allgather(g)
+                else:
+                    self._execute(g)
             except Exception as exc:  # surfaces in synchronize(), like a Status passed to the callback
                 for r, _ in g:
                     r.error = exc
@@ -190,20 +223,10 @@ class Engine:
     # ---- one fused response --------------------------------------------
 
     def _execute(self, group):
-        self.responses += 1
         first = group[0][0]
         tdt, wire = first.tensor_dtype, first.wire_dtype
         es = dtype_size(wire)
-        slot, self.slot = self.slot, (self.slot + 1) % len(self.streams)
-        s = self.streams[slot]
-        requests = []
-        for r, _ in group:
-            if r not in requests:
-                requests.append(r)
-        # the op's stream waits for the framework's stream(s), ops/nccl_operations.cc:140-154
-        for producer in {r.producer for r in requests}:
-            check(lib().hvdhip_stream_wait_event(s.handle, c_void_p(self.ready[producer].cuda_event)),
-                  "hvdhip_stream_wait_event")
+        slot, s, requests = self._begin(group)
         counts = [e.count for _, e in group]
         fused = len(group) > 1 or wire != tdt
         flags = PACK_CAST_THEN_SCALE if wire != tdt else 0
@@ -259,6 +282,59 @@ class Engine:
         marker = Marker(s, ev, len(requests))
         for r in requests:
             r.markers.append(marker)
+
+    def _begin(self, group):
+        """Picks the stream slot of a fused response and makes it wait for the framework."""
+        self.responses += 1
+        slot, self.slot = self.slot, (self.slot + 1) % len(self.streams)
+        s = self.streams[slot]
+        requests = []
+        for r, _ in group:
+            if r not in requests:
+                requests.append(r)
+        for producer in {r.producer for r in requests}:
+            check(lib().hvdhip_stream_wait_event(s.handle, c_void_p(self.ready[producer].cuda_event)),
+                  "hvdhip_stream_wait_event")
+        return slot, s, requests
+
+    def _finish(self, s, requests):
+        ev = c_void_p()  # completion marker from the event pool
+        check(lib().hvdhip_event_acquire(s.handle, ctypes.byref(ev)), "hvdhip_event_acquire")
+        check(lib().hvdhip_event_record(ev, s.handle), "hvdhip_event_record")
+        marker = Marker(s, ev, len(requests))
+        for r in requests:
+            r.markers.append(marker)
+
+    def _execute_allgather(self, group):
+        """The fusion-buffer side of a fused allgather (AllgatherOp::MemcpyInFusionBuffer /
+        MemcpyOutFusionBuffer, ops/collective_operations.cc:234-288): rank r's entries lie back
+        to back at displacement sum(recvcounts[:r]); entry e of rank r is copied out to row
+        offset sum(first dimensions of ranks < r) of output e.  Every rank's slab is packed here
+        (which stands in for the collective), each direction as one batched copy."""
+        slot, s, requests = self._begin(group)
+        es = dtype_size(group[0][0].tensor_dtype)
+        recv = [sum(e.parts[rank].numel() for _, e in group) * es for rank in range(self.size)]
+        total = sum(recv)
+        buf = self._buffer(slot, 0, total)
+        into_buf, from_src, nbytes, out_dst, from_buf = [], [], [], [], []
+        written = [0] * len(group)
+        at = 0
+        for rank in range(self.size):
+            for i, (_, e) in enumerate(group):
+                part = e.parts[rank]
+                n = part.numel() * es
+                if n:
+                    into_buf.append(buf + at)
+                    from_src.append(part.data_ptr())
+                    nbytes.append(n)
+                    out_dst.append(e.output.data_ptr() + written[i])
+                    from_buf.append(buf + at)
+                written[i] += n
+                at += n
+        if nbytes:
+            H.batched_d2d_memcpy(into_buf, from_src, nbytes, s)
+            H.batched_d2d_memcpy(out_dst, from_buf, nbytes, s)
+        self._finish(s, requests)
 
     @staticmethod
     def _scale_or_copy(src, dst, count, scale, dtype, s):

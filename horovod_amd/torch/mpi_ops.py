@@ -305,6 +305,65 @@ def grouped_allreduce_(tensors, average=None, name=None, op=None, prescale_facto
     return synchronize(grouped_allreduce_async_(tensors, average, name, op, prescale_factor, postscale_factor))
 
 
+def allgather_async(tensor, name=None):
+    """Asynchronously concatenates the tensor with the same-named tensor of every other rank along
+    the first dimension, which may differ between ranks (horovod/torch/mpi_ops.py:553-571)."""
+    eng = _state()
+    _check(tensor)
+    output = tensor.new()
+    req = Request([Entry(_name(name, 'allgather'), tensor, output)], SUM, 1.0, 1.0, 1, TORCH_TO_HVD[tensor.dtype],
+                  TORCH_TO_HVD[tensor.dtype], tensor.device.index, kind="allgather")
+    req.grouped = False
+    try:
+        eng.enqueue(req)
+    except RuntimeError as e:
+        raise e if isinstance(e, HorovodInternalError) else HorovodInternalError(e)
+    handle = _next_handle[0] = _next_handle[0] + 1
+    _handle_map[handle] = req
+    return handle
+
+
+class HorovodAllgather(torch.autograd.Function):
+    """The gradient of an allgather is this rank's rows of the averaged gradient
+    (horovod/torch/mpi_ops.py:574-592)."""
+
+    @staticmethod
+    def forward(ctx, tensor, name):
+        ctx.dim = tensor.shape[0] if tensor.dim() else 0
+        return synchronize(allgather_async(tensor.contiguous(), name))
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        grad_reduced = allreduce(grad_output.contiguous(), op=Average)
+        return grad_reduced.narrow(0, 0, ctx.dim), None  # this process is rank 0: its rows come first
+
+
+def allgather(tensor, name=None):
+    """Concatenation over ranks along the first dimension; differentiable."""
+    return HorovodAllgather.apply(tensor, name)
+
+
+def sparse_allreduce_async(tensor, name, op):
+    """A sparse gradient travels as two allgathers, of its indices (transposed, so that entries
+    concatenate along the first dimension) and of its values; duplicate indices stay uncoalesced
+    and add up when the result is used (horovod/torch/mpi_ops.py:515-535).  Returns a callable
+    that waits and builds the combined sparse tensor."""
+    t = tensor
+    indices_handle = allgather_async(t._indices().transpose(0, 1).contiguous(), name='%s.indices' % name)
+    values_handle = allgather_async(t._values().contiguous(), name='%s.values' % name)
+
+    def handle():
+        values = synchronize(values_handle)
+        indices = synchronize(indices_handle)
+        if op == Average:
+            values = values / size()
+        if indices.dim() == 0 or values.dim() == 0:
+            return t.new().resize_as_(t)
+        return torch.sparse_coo_tensor(indices.transpose(0, 1), values, t.size(), device=t.device)
+
+    return handle
+
+
 def poll(handle):
     """True once the operation behind the handle has completed on the GPU; does not block."""
     if handle not in _handle_map:

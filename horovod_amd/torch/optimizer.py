@@ -134,8 +134,8 @@ class _DistributedOptimizer(torch.optim.Optimizer):
         tensor = p.grad
         if tensor.is_sparse:
             if not self.sparse_as_dense:
-                raise NotImplementedError('sparse gradients travel by allgather, which this build does not drive; '
-                                          'pass sparse_as_dense=True')
+                # indices and values by allgather, optimizer.py:215-217
+                return mpi_ops.sparse_allreduce_async(tensor, name=name, op=self.op), None
             tensor = tensor.to_dense()
         pre, post = self._factors()
         if self._compression is Compression.fp16 and Compression.fp16.fuses_into_packing(tensor):
@@ -182,11 +182,11 @@ class _DistributedOptimizer(torch.optim.Optimizer):
 
     def _finish(self, p, output, ctx):
         self._allreduce_delay[p] = self.backward_passes_per_step
-        if ctx is None and output.data_ptr() == p.grad.data_ptr():
+        if ctx is None and not output.is_sparse and not p.grad.is_sparse and output.data_ptr() == p.grad.data_ptr():
             return  # reduced in place
-        result = self._compression.decompress(output, ctx)
+        result = output if ctx is None else self._compression.decompress(output, ctx)
         if p.grad.is_sparse:
-            p.grad.zero_().add_(result.to_sparse())
+            p.grad.zero_().add_(result if result.is_sparse else result.to_sparse())
         else:
             p.grad.set_(result)
 
@@ -207,7 +207,8 @@ class _DistributedOptimizer(torch.optim.Optimizer):
                 if self._groups is not None:
                     self._group_counts[p] = 0
             else:
-                output = mpi_ops.synchronize(handle)
+                # a sparse gradient's handle is a function that waits and assembles the result
+                output = handle() if callable(handle) else mpi_ops.synchronize(handle)
                 if self._groups is not None:
                     self._group_counts[self._p_to_group[p]] = 0
                 self._finish(p, output, ctx)

@@ -176,3 +176,26 @@ def test_adasum_optimizer_combines_deltas(hvd, orc):
         want = before[n].cpu().numpy().reshape(-1) + combined
         assert np.allclose(p.detach().cpu().numpy().reshape(-1), want, rtol=1e-6, atol=1e-8), n
     opt.zero_grad()
+
+
+@pytest.mark.parametrize("sparse_as_dense", [False, True])
+def test_sparse_gradients_travel_by_allgather(hvd, sparse_as_dense):
+    """An embedding with sparse=True: indices and values are allgathered (optimizer.py:215-217,
+    mpi_ops.py:515-535), or the gradient is densified first when sparse_as_dense is set."""
+    size = 2
+    hvd.init(size=size)
+    torch.manual_seed(8)
+    emb = torch.nn.Embedding(50, 8, sparse=True).cuda()
+    idx = torch.tensor([1, 7, 7, 33], device="cuda")
+    emb(idx).sum().backward()
+    local = emb.weight.grad.to_dense().clone()
+    emb.weight.grad = None
+    opt = hvd.DistributedOptimizer(torch.optim.SGD(emb.parameters(), lr=0.5), named_parameters=emb.named_parameters(),
+                                   sparse_as_dense=sparse_as_dense)
+    before = emb.weight.detach().clone()
+    emb(idx).sum().backward()
+    assert emb.weight.grad.is_sparse
+    opt.step()
+    # every rank holds the same gradient: the average is that gradient
+    assert torch.allclose(emb.weight.grad.to_dense(), local)
+    assert torch.allclose(emb.weight, before - 0.5 * local)
