@@ -418,6 +418,55 @@ def extras(steps, warmup):
                                          "replicas_rotated": len(pairs)}
     plan.destroy()
     del pairs
+    torch.cuda.empty_cache()
+
+    # Allgather fusion buffer (ops/collective_operations.cc:234-288): 8 ranks, 128 entries per rank with
+    # the stress workload's size mix.  This GPU packs its own slab at its displacement (the other
+    # slabs arrive by the collective, which is not built) and unpacks one component per (entry, rank).
+    # Each direction is one batched copy; 4 independent sets are rotated.
+    import ctypes
+    import horovod_amd
+    world, es = 8, 4
+    counts = W.stress_counts(seed=21, n=128)
+    slab = es * sum(counts)
+    sets = []
+    for r in range(4):
+        src = DeviceSet(counts, es, lambda n: randn(n, torch.float32, 1.0, 60 + r))
+        fusion = torch.empty(world * slab, dtype=torch.uint8, device="cuda")
+        outs = [torch.empty(world * c * es, dtype=torch.uint8, device="cuda") for c in counts]
+        pack_dst, at = [], 3 * slab  # this rank's displacement (rank 3 of 8)
+        for c in counts:
+            pack_dst.append(fusion.data_ptr() + at)
+            at += c * es
+        un_dst, un_src, un_sz = [], [], []
+        for rank in range(world):
+            at = rank * slab
+            for i, c in enumerate(counts):
+                un_dst.append(outs[i].data_ptr() + rank * c * es)
+                un_src.append(fusion.data_ptr() + at)
+                un_sz.append(c * es)
+                at += c * es
+        # the descriptor arrays as the C caller holds them, built once
+        VP, SZ = ctypes.c_void_p, ctypes.c_size_t
+        pack_args = ((VP * len(counts))(*pack_dst), (VP * len(counts))(*src.ptrs),
+                     (SZ * len(counts))(*[c * es for c in counts]), len(counts))
+        un_args = ((VP * len(un_dst))(*un_dst), (VP * len(un_dst))(*un_src), (SZ * len(un_dst))(*un_sz), len(un_dst))
+        sets.append((src, fusion, outs, pack_args, un_args))
+    torch.cuda.synchronize()
+    copy = horovod_amd.lib().hvdhip_batched_d2d_memcpy
+
+    def gather_step():
+        i = turn[0] = (turn[0] + 1) % len(sets)
+        horovod_amd.check(copy(*sets[i][3], s.handle), "hvdhip_batched_d2d_memcpy")
+        horovod_amd.check(copy(*sets[i][4], s.handle), "hvdhip_batched_d2d_memcpy")
+
+    sec = event_timed(gather_step, s, max(8, steps // 4), 4)
+    ab = 2 * slab + 2 * world * slab
+    out["allgather_fusion_8ranks_pack_unpack"] = {
+        "GB/s": round(ab / sec / 1e9, 1), "frac_of_hbm_peak": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4),
+        "ms": round(sec * 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1), "entries": len(counts), "ranks": world,
+        "copies_per_step": len(counts) * (world + 1), "streams": 1, "replicas_rotated": len(sets)}
+    del sets
     return out
 
 
