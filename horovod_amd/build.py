@@ -1,4 +1,5 @@
-"""Builds the in-tree native libraries with make (hipcc for gfx950, g++ for the adapter)."""
+"""Builds the in-tree native libraries with make (hipcc for gfx950, g++ for the adapter, gcc for the
+C99 example client)."""
 import os
 import subprocess
 
@@ -16,6 +17,6 @@ def build(force=False, jobs=8):
 
 def ensure_built():
     """Builds the libraries only if one of them is missing; never replaces an existing build."""
-    need = [os.path.join(_HERE, "lib", n) for n in ("libhvdhip.so", "libhvdhip_adapter.so")]
+    need = [os.path.join(_HERE, "lib", n) for n in ("libhvdhip.so", "libhvdhip_adapter.so", "c_client")]
     if not all(os.path.exists(p) for p in need):
         build()
