@@ -161,10 +161,6 @@ def reduce_sum_k(resident_ptr, incoming_ptrs, n, dtype, stream):
                                     stream.handle), "hvdhip_reduce_sum_k")
 
 
-__all__ = ["Stream", "Timer", "FusionPlan", "AdasumPlan", "batched_d2d_memcpy", "batched_scaled_d2d_memcpy",
-           "scale_buffer", "reduce_sum", "reduce_sum_k", "DTYPE"]
-
-
 FP16_SCALE_FP32_FACTOR = 0  # ScaleBufferCPUImpl<unsigned short, float>, ops/collective_operations.h:99-127
 FP16_SCALE_HALF_FACTOR = 1  # scale_buffer_k<__half>, ops/cuda/cuda_kernels.cu:96-136,167
 
@@ -175,3 +171,8 @@ def set_fp16_scale_mode(mode):
 
 def get_fp16_scale_mode():
     return int(lib().hvdhip_get_fp16_scale_mode())
+
+
+__all__ = ["Stream", "Timer", "FusionPlan", "AdasumPlan", "batched_d2d_memcpy", "batched_scaled_d2d_memcpy",
+           "scale_buffer", "reduce_sum", "reduce_sum_k", "DTYPE", "FP16_SCALE_FP32_FACTOR", "FP16_SCALE_HALF_FACTOR",
+           "set_fp16_scale_mode", "get_fp16_scale_mode"]

@@ -19,7 +19,7 @@ import ctypes
 import torch
 
 from . import host as H
-from ._lib import DTYPE, check, dtype_size, lib
+from ._lib import check, dtype_size, lib
 from .workloads import FUSION_THRESHOLD, fuse
 
 

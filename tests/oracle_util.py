@@ -5,7 +5,7 @@ The oracle is the checker only: nothing here is used by the library under test.
 import ctypes
 import os
 import subprocess
-from ctypes import POINTER, c_double, c_float, c_int, c_int64, c_void_p
+from ctypes import c_double, c_float, c_int, c_int64, c_void_p
 
 import numpy as np
 

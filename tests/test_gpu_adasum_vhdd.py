@@ -12,7 +12,6 @@ scaled_add) at exactly the slice shapes and per-slice layer counts a rank would 
 result must equal the pairwise tree that the oracle computes on whole vectors."""
 import numpy as np
 import pytest
-import torch
 
 from oracle_util import F16, F32, NP_OF, SIZE_OF
 
