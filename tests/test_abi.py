@@ -81,3 +81,50 @@ def test_c_client_is_built_with_the_library():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     assert os.path.exists(os.path.join(root, "horovod_amd", "lib", "c_client")), \
         "make -C horovod_amd/csrc builds the C99 example next to the library"
+
+
+def test_more_argument_errors_are_caught_before_the_device_is_touched():
+    """Validation comes first in every entry point, so these calls must fail the same way on a
+    machine without a GPU."""
+    import horovod_amd
+    L = horovod_amd.lib()
+    D = horovod_amd.DTYPE
+    one = (ctypes.c_void_p * 1)(16)
+    cnt = (ctypes.c_int64 * 1)(-4)
+    plan = ctypes.c_void_p()
+    # a negative element count
+    assert L.hvdhip_fusion_plan_create(one, one, cnt, 1, D["float32"], D["float32"], ctypes.byref(plan)) == -1
+    assert b"negative" in L.hvdhip_last_error()
+    cnt[0] = 4
+    # only float32 tensors may travel in a float16 buffer
+    assert L.hvdhip_fusion_plan_create(one, one, cnt, 1, D["int32"], D["float16"], ctypes.byref(plan)) == -2
+    assert L.hvdhip_fusion_plan_create(one, one, cnt, 1, D["float16"], D["float32"], ctypes.byref(plan)) == -2
+    assert L.hvdhip_fusion_plan_create(one, one, cnt, 1, 42, 42, ctypes.byref(plan)) == -2
+    # misaligned for its element size
+    odd = (ctypes.c_void_p * 1)(18)
+    assert L.hvdhip_fusion_plan_create(odd, one, cnt, 1, D["float32"], D["float32"], ctypes.byref(plan)) == -1
+    assert b"aligned" in L.hvdhip_last_error()
+    # a NULL tensor with elements in it
+    null = (ctypes.c_void_p * 1)(None)
+    assert L.hvdhip_fusion_plan_create(null, one, cnt, 1, D["float32"], D["float32"], ctypes.byref(plan)) == -1
+    assert L.hvdhip_fusion_plan_create(one, one, cnt, 1, D["float32"], D["float32"], None) == -1
+    # pack / unpack / reduce / Adasum without a plan or with impossible arguments
+    assert L.hvdhip_fusion_pack(None, None, 1.0, 0, None) == -1
+    assert L.hvdhip_fusion_unpack(None, None, 1.0, None) == -1
+    assert L.hvdhip_fusion_plan_buffer_len(None) == -1 and L.hvdhip_fusion_plan_num_chunks(None) == -1
+    assert L.hvdhip_reduce_sum(None, None, -1, D["float32"], None) == -1
+    assert L.hvdhip_reduce_sum(None, None, 0, D["bool"], None) == -2
+    ad = ctypes.c_void_p()
+    neg = (ctypes.c_int * 2)(5, -1)
+    assert L.hvdhip_adasum_plan_create(neg, 2, D["float32"], ctypes.byref(ad)) == -1
+    assert L.hvdhip_adasum_plan_create(neg, 2, D["int32"], ctypes.byref(ad)) == -2
+    assert L.hvdhip_adasum_combine(None, None, None, None) == -1
+    assert L.hvdhip_adasum_dispatch_scaled_add(D["float32"], -3, 1.0, None, 1.0, None, None) == -1
+    sizes = (ctypes.c_size_t * 1)(6)
+    assert L.hvdhip_batched_d2d_memcpy(one, one, sizes, -1, None) == -1
+    assert L.hvdhip_batched_scaled_d2d_memcpy(one, one, sizes, 1, 0.5, D["float32"], None) == -1  # 6 is no multiple of 4
+    assert L.hvdhip_batched_scaled_d2d_memcpy(one, one, sizes, 1, 0.5, D["bool"], None) == -2
+    assert L.hvdhip_set_fp16_scale_mode(3) == -1 and L.hvdhip_get_fp16_scale_mode() == 0
+    assert L.hvdhip_memcpy_async(None, None, 0, 9, None) == -1
+    for code in (-1, -2, -3, -4, 1, 2, 700):
+        assert L.hvdhip_error_string(code)
