@@ -34,7 +34,9 @@ namespace hvdhip {
 namespace {
 
 // Chunk table entry as used here: tensor = index of the chunk's first element
-// in the vectors, output = layer number, n = elements in the chunk.
+// in the vectors, output = layer number, off = the chunk's number in layer order
+// (the slot of its partial triple; the table itself is in XCD order), n = elements
+// in the chunk.
 //
 // Layer table entry: first partial triple of the layer and how many it has.
 struct Layer {
@@ -133,9 +135,9 @@ __global__ __launch_bounds__(kWG) void dot_partials_k(const Chunk* __restrict__ 
   }
   Triple r = wg_reduce(Triple{d0 + d1, a0 + a1, b0 + b1});
   if (threadIdx.x == 0) {
-    partials[3 * (uint64_t)blockIdx.x + 0] = r.d;
-    partials[3 * (uint64_t)blockIdx.x + 1] = r.a;
-    partials[3 * (uint64_t)blockIdx.x + 2] = r.b;
+    partials[3 * c.off + 0] = r.d;  // c.off: the chunk's number in layer order, whatever workgroup has it
+    partials[3 * c.off + 1] = r.a;
+    partials[3 * c.off + 2] = r.b;
   }
 }
 
@@ -247,7 +249,7 @@ __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ ch
       layer_coeffs(r, guard, &ca, &cb);
       cc[0] = ca;
       cc[1] = cb;
-      if (blockIdx.x == L.first) {
+      if (c.off == L.first) {
         normdots[3 * c.output + 0] = r.d;
         normdots[3 * c.output + 1] = r.a;
         normdots[3 * c.output + 2] = r.b;
@@ -466,7 +468,8 @@ int hvdhip_adasum_plan_create(const int* tensor_counts, int nlayers, int dtype,
     layers[(size_t)i].first = (uint32_t)chunks.size();
     for (uint64_t start = 0; start < n; start += chunk_units) {
       const uint64_t left = n - start;
-      chunks.push_back(Chunk{off + start, (uint64_t)i, 0, (uint32_t)(left < chunk_units ? left : chunk_units), 0});
+      chunks.push_back(Chunk{off + start, (uint64_t)i, (uint64_t)chunks.size(),
+                             (uint32_t)(left < chunk_units ? left : chunk_units), 0});
     }
     layers[(size_t)i].count = (uint32_t)chunks.size() - layers[(size_t)i].first;
     if (layers[(size_t)i].count > max_layer_chunks) max_layer_chunks = layers[(size_t)i].count;
@@ -479,6 +482,11 @@ int hvdhip_adasum_plan_create(const int* tensor_counts, int nlayers, int dtype,
   p->total = (int64_t)off;
   p->max_layer_chunks = max_layer_chunks;
   (void)hipGetDevice(&p->device);
+  {
+    std::vector<Chunk> ordered(chunks.size());
+    for (size_t c = 0; c < chunks.size(); ++c) ordered[xcd_slot(c, chunks.size(), xcd_run(chunks.size()))] = chunks[c];
+    chunks.swap(ordered);
+  }
   int rc = upload_chunks(chunks, &p->tables);
   if (rc) {
     delete p;

@@ -103,8 +103,26 @@ uint64_t count_chunks(const std::vector<Seg>& segs, uint32_t chunk_units) {
   return nchunks > kMaxWorkgroups ? ~0ull : nchunks;
 }
 
+uint32_t xcd_run(uint64_t nchunks) {
+  static const uint32_t run = [] {
+    const char* e = std::getenv("HVDHIP_XCD_RUN");
+    return e ? (uint32_t)std::strtoul(e, nullptr, 10) : kXcdRun;
+  }();
+  return nchunks > kXcdOrderMaxChunks ? 0 : run;
+}
+
+uint32_t xcd_shift(uint64_t nblocks) {
+  const uint32_t run = xcd_run(nblocks);
+  if (run == 0 || (run & (run - 1)) != 0) return kNoXcdOrder;
+  uint32_t shift = 0;
+  while ((1u << shift) < run) ++shift;
+  return shift;
+}
+
 void fill_chunks(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t tensor_es,
-                 uint32_t buffer_es, Chunk* out) {
+                 uint32_t buffer_es, Chunk* out, uint64_t nchunks) {
+  const uint32_t run = xcd_run(nchunks);
+  uint64_t index = 0;
   for (const Seg& s : segs) {
     const uint64_t nbytes = s.n * buffer_es;
     for (uint64_t start = 0; start < s.n; start += chunk_units) {
@@ -115,7 +133,7 @@ void fill_chunks(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t te
       c.off = s.off + start * buffer_es;
       c.n = (uint32_t)(left < chunk_units ? left : chunk_units);
       c.pad = left <= chunk_units ? (uint32_t)((16 - (nbytes & 15)) & 15) : 0;
-      *out++ = c;
+      out[xcd_slot(index++, nchunks, run)] = c;
     }
   }
 }
@@ -126,7 +144,7 @@ int build_tables(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t te
   const uint64_t nchunks = count_chunks(segs, chunk_units);
   if (nchunks == ~0ull) return fail(HVDHIP_ERR_TOO_LARGE, "plan needs more than 2^23 workgroups");
   std::vector<Chunk> chunks((size_t)nchunks);
-  fill_chunks(segs, chunk_units, tensor_es, buffer_es, chunks.data());
+  fill_chunks(segs, chunk_units, tensor_es, buffer_es, chunks.data(), nchunks);
   return upload_chunks(chunks, out);
 }
 

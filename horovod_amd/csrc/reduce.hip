@@ -38,13 +38,13 @@ struct Peers {
 
 constexpr int kUnroll = 2;
 
-// Workgroup b accumulates K peers into elements [b*tile, (b+1)*tile).
+// Workgroup b accumulates K peers into tile t = xcd_tile(b), elements [t*tile, (t+1)*tile).
 template <typename T, int K>
 __global__ __launch_bounds__(kWG) void reduce_k(T* resident, Peers<K> peers, uint64_t n,
-                                                uint32_t tile) {
+                                                uint32_t tile, uint32_t run) {
   constexpr int VEC = 16 / (int)sizeof(T);
   typedef Arr<T, VEC> V;
-  const uint64_t start = (uint64_t)blockIdx.x * tile;
+  const uint64_t start = (uint64_t)xcd_tile(blockIdx.x, gridDim.x, run) * tile;
   const uint64_t left = n - start;
   const uint32_t m = left < tile ? (uint32_t)left : tile;
   gptr<T> r = as_global(resident + start);
@@ -100,7 +100,7 @@ int launch_k(void* resident, const void* const* incoming, int64_t n, hipStream_t
     Peers<K> peers;
     for (int k = 0; k < K; ++k) peers.p[k] = static_cast<const T*>(incoming[k]) + done;
     hipLaunchKernelGGL((reduce_k<T, K>), dim3(blocks), dim3(kWG), 0, stream, static_cast<T*>(resident) + done,
-                       peers, slice, tile);
+                       peers, slice, tile, xcd_shift(blocks));
     HVDHIP_CHECK_LAUNCH("reduce_k");
     done += slice;
     left -= slice;

@@ -182,12 +182,12 @@ __global__ __launch_bounds__(kWG) void xfer_k(const Chunk* __restrict__ chunks, 
     as_global<uint8_t>(dst_addr)[(uint64_t)c.n * sizeof(D) + threadIdx.x] = 0;
 }
 
-// Contiguous buffer: workgroup b handles elements [b*tile, (b+1)*tile).
+// Contiguous buffer: workgroup b handles tile t = xcd_tile(b), elements [t*tile, (t+1)*tile).
 template <class Op>
 __global__ __launch_bounds__(kWG) void contig_k(const typename Op::S* src,
                                                 typename Op::D* dst, uint64_t n,
-                                                uint32_t tile, typename Op::P p) {
-  const uint64_t start = (uint64_t)blockIdx.x * tile;
+                                                uint32_t tile, uint32_t run, typename Op::P p) {
+  const uint64_t start = (uint64_t)xcd_tile(blockIdx.x, gridDim.x, run) * tile;
   const uint64_t left = n - start;
   const uint32_t m = left < tile ? (uint32_t)left : tile;
   stream_range<Op>(as_global(src + start), as_global(dst + start), m, p);
@@ -251,7 +251,7 @@ int launch_contig(const void* in, void* out, int64_t n, typename Op::P p, hipStr
   while (left > 0) {  // one launch unless the buffer needs more than kMaxWorkgroups workgroups
     const uint64_t slice = std::min<uint64_t>(left, kMaxWorkgroups * tile);
     const uint32_t blocks = (uint32_t)((slice + tile - 1) / tile);
-    hipLaunchKernelGGL((contig_k<Op>), dim3(blocks), dim3(kWG), 0, stream, src, dst, slice, tile, p);
+    hipLaunchKernelGGL((contig_k<Op>), dim3(blocks), dim3(kWG), 0, stream, src, dst, slice, tile, xcd_shift(blocks), p);
     HVDHIP_CHECK_LAUNCH("contig_k");
     src += slice;
     dst += slice;
@@ -393,7 +393,7 @@ int cached_tables(void* const* out, const void* const* in, const size_t* sizes, 
   if (rc) return rc;
   hipError_t e = hipEventCreateWithFlags(&entry.done, hipEventDisableTiming);
   if (e == hipSuccess && nchunks) {
-    fill_chunks(segs, chunk_units, unit, unit, static_cast<Chunk*>(entry.buf.pinned));
+    fill_chunks(segs, chunk_units, unit, unit, static_cast<Chunk*>(entry.buf.pinned), nchunks);
     e = hipMemcpyAsync(entry.buf.dev, entry.buf.pinned, bytes, hipMemcpyHostToDevice, stream);
   }
   if (e != hipSuccess) {

@@ -129,3 +129,23 @@ def test_reduce_rejects_bool_and_bad_k(gpu):
     assert e.value.code == -2
     with pytest.raises(horovod_amd.HvdHipError):
         gpu.H.reduce_sum_k(t.data_ptr(), [t.data_ptr()] * 17, 4, F32, gpu.stream)
+
+
+@pytest.mark.parametrize("dtype", [F32, F16])
+@pytest.mark.parametrize("n_tiles", [512, 513, 1024 + 300, 5 * 512 + 1])
+def test_tile_order_across_xcd_groups(gpu, orc, dtype, n_tiles):
+    """Contiguous kernels hand tiles to workgroups in groups of 512 so that each XCD walks runs of 64
+    consecutive tiles, and leave a ragged last group in natural order: whole groups, a group plus
+    one tile, and sizes that end inside a tile must all give the oracle's values."""
+    rng = np.random.default_rng(n_tiles)
+    es = SIZE_OF[dtype]
+    n = n_tiles * (4096 // es) - 37
+    v = _vals(rng, n, dtype, 1e-2 if dtype == F16 else 1.0)
+    p = _vals(rng, n, dtype, 1e-2 if dtype == F16 else 1.0)
+    d_v, d_p, d_o = gpu.upload(_raw(v)), gpu.upload(_raw(p)), gpu.empty(n * es + 64, fill=0x5A)
+    gpu.H.scale_buffer(d_v.data_ptr(), d_o.data_ptr(), n, 0.125, dtype, gpu.stream)
+    out = gpu.download(d_o)
+    assert np.array_equal(out[:n * es], orc.scale_buffer(_raw(v), 0.125, dtype).view(np.uint8))
+    assert np.all(out[n * es:] == 0x5A)
+    gpu.H.reduce_sum(d_v.data_ptr(), d_p.data_ptr(), n, dtype, gpu.stream)
+    assert np.array_equal(gpu.download(d_v)[:n * es], orc.sum(_raw(p), _raw(v), dtype).view(np.uint8))
