@@ -104,11 +104,12 @@ uint64_t count_chunks(const std::vector<Seg>& segs, uint32_t chunk_units) {
 }
 
 uint32_t xcd_run(uint64_t nchunks) {
-  static const uint32_t run = [] {
+  static const long forced = [] {
     const char* e = std::getenv("HVDHIP_XCD_RUN");
-    return e ? (uint32_t)std::strtoul(e, nullptr, 10) : kXcdRun;
+    return e ? std::strtol(e, nullptr, 10) : -1L;
   }();
-  return nchunks > kXcdOrderMaxChunks ? 0 : run;
+  if (forced >= 0) return (uint32_t)forced;
+  return nchunks <= kXcdLongRunFrom ? kXcdRun : kXcdLongRun;
 }
 
 uint32_t xcd_shift(uint64_t nblocks) {

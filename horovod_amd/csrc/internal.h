@@ -83,14 +83,15 @@ uint32_t chunk_bytes(Family f);
 // (1.5-2.5 % on the pack and unpack kernels, up to 5 % on the widening unpack) when one XCD walks
 // runs of consecutive chunks instead of every eighth chunk, so tables and tile numbers are laid out
 // accordingly: within each group of 8 * run chunks, XCD x gets chunks x * run .. x * run + run - 1.
-// The ragged end (fewer than 8 * run chunks) keeps its natural order.  Measured best at run = 64
-// (32-256 are close) for launches of up to 128 MiB, +2-5 % on every kernel family; launches of
-// 512 MiB and more lose with that run length (-2 % scale, -6 % reduce), so launches of more than
-// kXcdOrderMaxChunks chunks keep the natural order.  HVDHIP_XCD_RUN overrides the run length,
-// 0 switches the reordering off.
+// The ragged end (fewer than 8 * run chunks) keeps its natural order.  Measured against natural
+// order: runs of 64 chunks are best for launches of 16-128 MiB (+2-5 % on every kernel family; 32-256
+// are close, 1 and >= 1,024 gain nothing) but cost 2-6 % at 512 MiB and more, where runs of 256 gain
+// 1-3 %; so launches of more than kXcdLongRunFrom chunks use the longer run.  HVDHIP_XCD_RUN
+// overrides the run length for every launch, 0 switches the reordering off.
 constexpr uint32_t kXcds = 8;
 constexpr uint32_t kXcdRun = 64;
-constexpr uint64_t kXcdOrderMaxChunks = 65536;  // 256 MiB of 4 KiB chunks
+constexpr uint32_t kXcdLongRun = 256;
+constexpr uint64_t kXcdLongRunFrom = 32768;  // 128 MiB of 4 KiB chunks
 uint32_t xcd_run(uint64_t nchunks);
 // Chunk (or tile) that the workgroup at table position `slot` handles.
 __host__ __device__ inline uint64_t xcd_chunk(uint64_t slot, uint64_t nchunks, uint32_t run) {
