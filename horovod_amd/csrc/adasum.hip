@@ -498,6 +498,8 @@ int hvdhip_adasum_plan_create(const int* tensor_counts, int nlayers, int dtype,
   if (e == hipSuccess) e = hipMemset(p->results, 0, ndoubles * sizeof(double));
   if (e == hipSuccess && nlayers > 0)
     e = hipMemcpy(p->results + ndoubles, layers.data(), layer_bytes, hipMemcpyHostToDevice);
+  // the fill above may return before the device has done it; the plan is used on other streams
+  if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
   if (e != hipSuccess) {
     (void)hipGetLastError();
     if (p->results) (void)hipFree(p->results);
@@ -516,7 +518,8 @@ int hvdhip_adasum_plan_create(const int* tensor_counts, int nlayers, int dtype,
 
 int hvdhip_adasum_plan_destroy(hvdhip_adasum_plan* plan) {
   if (!plan) return ok();
-  HVDHIP_CHECK(hipDeviceSynchronize());
+  DeviceGuard on_plan_device(plan->device);
+  HVDHIP_CHECK(hipDeviceSynchronize());  // queued kernels may still read the tables
   int rc = free_tables(&plan->tables);
   if (plan->results) (void)hipFree(plan->results);
   delete plan;

@@ -258,12 +258,12 @@ int hvdhip_event_acquire(void* stream, void** event) {
     auto key = std::make_pair(dev, s);
     auto& q = p.idle[key];
     if (!p.filled[key]) {
+      p.filled[key] = true;  // one attempt per stream, also when it stops early on an error
       for (int i = 0; i < kPrepopulate; ++i) {
         hipEvent_t ev;
         HVDHIP_CHECK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
         q.push_back(ev);
       }
-      p.filled[key] = true;
     }
     if (!q.empty()) {
       *event = q.back();

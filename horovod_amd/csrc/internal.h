@@ -161,6 +161,25 @@ int build_tables(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t te
 uint64_t count_chunks(const std::vector<Seg>& segs, uint32_t chunk_units);
 void fill_chunks(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t tensor_es,
                  uint32_t buffer_es, Chunk* out, uint64_t nchunks);
+// Makes `device` current for its lifetime when another one is, and puts the old one back.
+// Plans and cached tables belong to the device that was current when they were made; their
+// teardown must wait for and free on that device whatever the caller has selected since.
+class DeviceGuard {
+ public:
+  explicit DeviceGuard(int device) {
+    if (hipGetDevice(&prev_) == hipSuccess && prev_ != device && hipSetDevice(device) == hipSuccess) switched_ = true;
+  }
+  ~DeviceGuard() {
+    if (switched_) (void)hipSetDevice(prev_);
+  }
+  DeviceGuard(const DeviceGuard&) = delete;
+  DeviceGuard& operator=(const DeviceGuard&) = delete;
+
+ private:
+  int prev_ = 0;
+  bool switched_ = false;
+};
+
 // Uploads a ready-made chunk table.
 int upload_chunks(const std::vector<Chunk>& chunks, DevTables* out);
 int free_tables(DevTables* t);

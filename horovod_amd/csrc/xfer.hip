@@ -27,6 +27,7 @@
 #include <algorithm>
 #include <cstring>
 #include <list>
+#include <map>
 #include <mutex>
 
 #include "internal.h"
@@ -278,7 +279,7 @@ struct TableBuf {
 };
 
 struct CachedCopy {
-  std::vector<uint64_t> key;  // device and unit size, n, then out/in/size triples
+  std::vector<uint64_t> key;  // unit size, n, then out/in/size triples
   DevTables tables;           // tables.alloc is not owned: it aliases buf.dev
   TableBuf buf;
   hipEvent_t done = nullptr;        // recorded after every launch that reads the table
@@ -286,14 +287,23 @@ struct CachedCopy {
   bool several_streams = false;     // used on more than one stream since it was built
 };
 
+// One cache per device: its entries, their buffers and the spare buffers all live on that
+// device, and it is only ever touched with that device current.
 struct CopyCache {
   std::mutex mu;
   std::list<CachedCopy> lru;  // front = most recent
   std::vector<TableBuf> spare;
 };
-CopyCache& copy_cache() {
-  static CopyCache* c = new CopyCache();
-  return *c;
+int copy_cache(CopyCache** out) {
+  static std::mutex mu;
+  static std::map<int, CopyCache*>* caches = new std::map<int, CopyCache*>();  // never destroyed
+  int device = 0;
+  HVDHIP_CHECK(hipGetDevice(&device));
+  std::lock_guard<std::mutex> g(mu);
+  CopyCache*& c = (*caches)[device];
+  if (!c) c = new CopyCache();
+  *out = c;
+  return 0;
 }
 constexpr size_t kCopyCacheCapacity = 64;
 constexpr size_t kSpareBufs = 8;
@@ -352,20 +362,17 @@ int evict_one(CopyCache& c) {
 // Finds or builds the table for (out, in, sizes) with elements of unit bytes; a newly
 // built table is uploaded asynchronously on `stream`.  The caller holds the cache mutex,
 // launches on `stream`, then calls mark_used() before releasing the mutex.
-int cached_tables(void* const* out, const void* const* in, const size_t* sizes, int n,
+int cached_tables(CopyCache& c, void* const* out, const void* const* in, const size_t* sizes, int n,
                   uint32_t unit, hipStream_t stream, CachedCopy** result) {
-  int device = 0;
-  HVDHIP_CHECK(hipGetDevice(&device));
   std::vector<uint64_t> key;
   key.reserve(2 + 3 * (size_t)n);
-  key.push_back(((uint64_t)(uint32_t)device << 32) | unit);  // tables live on the device that built them
+  key.push_back((uint64_t)unit);
   key.push_back((uint64_t)n);
   for (int i = 0; i < n; ++i) {
     key.push_back((uint64_t)(uintptr_t)out[i]);
     key.push_back((uint64_t)(uintptr_t)in[i]);
     key.push_back((uint64_t)sizes[i]);
   }
-  CopyCache& c = copy_cache();
   for (auto it = c.lru.begin(); it != c.lru.end(); ++it) {
     if (it->key == key) {
       c.lru.splice(c.lru.begin(), c.lru, it);
@@ -438,6 +445,7 @@ using namespace hvdhip;
 
 struct hvdhip_fusion_plan {
   int n = 0;
+  int device = 0;  // the device that holds the tables
   int tensor_dtype = 0;
   int buffer_dtype = 0;
   int64_t buffer_len = 0;
@@ -456,8 +464,11 @@ int hvdhip_batched_d2d_memcpy(void* const* out, const void* const* in, const siz
   if (num_copies == 0) return ok();
   hipStream_t s = static_cast<hipStream_t>(stream);
   CachedCopy* entry = nullptr;
-  std::lock_guard<std::mutex> g(copy_cache().mu);
-  rc = cached_tables(out, in, sizes, num_copies, 1, s, &entry);
+  CopyCache* cache = nullptr;
+  rc = copy_cache(&cache);
+  if (rc) return rc;
+  std::lock_guard<std::mutex> g(cache->mu);
+  rc = cached_tables(*cache, out, in, sizes, num_copies, 1, s, &entry);
   if (rc) return rc;
   rc = launch_xfer<Copy<uint8_t>, kDirect>(entry->tables, 0, {}, s);
   int rc2 = mark_used(entry, s);
@@ -482,8 +493,11 @@ int hvdhip_batched_scaled_d2d_memcpy(void* const* out, const void* const* in,
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   CachedCopy* entry = nullptr;
-  std::lock_guard<std::mutex> g(copy_cache().mu);
-  rc = cached_tables(out, in, sizes, num_copies, es, s, &entry);
+  CopyCache* cache = nullptr;
+  rc = copy_cache(&cache);
+  if (rc) return rc;
+  std::lock_guard<std::mutex> g(cache->mu);
+  rc = cached_tables(*cache, out, in, sizes, num_copies, es, s, &entry);
   if (rc) return rc;
   rc = launch_same_dtype<kDirect>(entry->tables, 0, scale_factor, dtype, s);
   int rc2 = mark_used(entry, s);
@@ -554,6 +568,7 @@ int hvdhip_fusion_plan_create(const void* const* tensors, void* const* outputs,
   p->buffer_len = off;
   p->offsets.swap(offsets);
   p->converting = buffer_dtype != tensor_dtype;
+  (void)hipGetDevice(&p->device);
   // Chunks are sized on the wider (tensor) side.  The narrowing pack stores only 8 bytes per
   // lane and access and streams best with 8 KiB of fp32 per workgroup; the widening unpack and
   // every same-width transfer with 4 KiB.
@@ -574,6 +589,7 @@ int hvdhip_fusion_plan_create(const void* const* tensors, void* const* outputs,
 
 int hvdhip_fusion_plan_destroy(hvdhip_fusion_plan* plan) {
   if (!plan) return ok();
+  DeviceGuard on_plan_device(plan->device);
   // Queued kernels may still read the tables.
   HVDHIP_CHECK(hipDeviceSynchronize());
   int rc = free_tables(&plan->tables);

@@ -37,15 +37,13 @@ class FP16Compressor(Compressor):
 
     @staticmethod
     def compress(tensor):
-        if tensor.dtype.is_floating_point:
-            return tensor.type(torch.float16), tensor.dtype
-        return tensor, tensor.dtype
+        # the context is the dtype to come back to
+        travels = tensor.to(torch.float16) if tensor.dtype.is_floating_point else tensor
+        return travels, tensor.dtype
 
     @staticmethod
     def decompress(tensor, ctx):
-        if ctx.is_floating_point:
-            return tensor.type(ctx)
-        return tensor
+        return tensor.to(ctx) if ctx.is_floating_point else tensor
 
     @staticmethod
     def fuses_into_packing(tensor):

@@ -199,3 +199,137 @@ def test_sparse_gradients_travel_by_allgather(hvd, sparse_as_dense):
     # every rank holds the same gradient: the average is that gradient
     assert torch.allclose(emb.weight.grad.to_dense(), local)
     assert torch.allclose(emb.weight, before - 0.5 * local)
+
+
+def test_force_allreduce_on_parameters_without_gradient(hvd):
+    """test/parallel/test_torch.py:1791-1858: a branch of the model that this rank's loss does
+    not reach still takes part in step(): the rank contributes zeros (optimizer.py:174-181)."""
+    size = 2
+
+    def peer(rank, name, tensor):
+        return torch.full_like(tensor, 0.5)
+
+    hvd.init(size=size, peer_source=peer)
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc1 = torch.nn.Linear(10, 6)
+            self.fc2 = torch.nn.Linear(6, 4)
+            self.fc3 = torch.nn.Linear(4, 4)
+
+        def forward(self, x):
+            h = torch.relu(self.fc1(x))
+            a = self.fc2(h)
+            return a, self.fc3(torch.relu(a))
+
+    for cls, kwargs in [(torch.optim.SGD, dict(lr=0.2, momentum=0.9, weight_decay=0.1)), (torch.optim.Adam, dict(lr=0.2)),
+                        (torch.optim.RMSprop, dict(lr=0.2, centered=True)), (torch.optim.Adagrad, dict(lr=0.2))]:
+        torch.manual_seed(5)
+        model = Net().cuda()
+        opt = hvd.DistributedOptimizer(cls(model.parameters(), **kwargs), named_parameters=model.named_parameters())
+        assert isinstance(opt, cls)
+        first, _ = model(torch.randn(8, 10, device="cuda"))
+        opt.zero_grad()
+        first.pow(2).sum().backward()  # fc3 gets no gradient here
+        assert model.fc3.weight.grad is None
+        opt.synchronize()
+        # zeros from this rank and 0.5 from the other, averaged
+        assert torch.equal(model.fc3.weight.grad, torch.full_like(model.fc3.weight, 0.25)), cls.__name__
+        assert torch.equal(model.fc3.bias.grad, torch.full_like(model.fc3.bias, 0.25)), cls.__name__
+        with opt.skip_synchronize():
+            opt.step()
+        assert all(torch.isfinite(p).all() for p in model.parameters())
+
+
+def test_dynamic_requires_grad(hvd):
+    """test/parallel/test_torch.py:1961-2009: two optimizers whose parameters are switched off and
+    on between steps; only the trained half gets (non-zero) gradients and only its optimizer steps."""
+    hvd.init(size=2)
+    torch.manual_seed(6)
+    gen = torch.nn.Conv2d(1, 10, 1).cuda()
+    disc = torch.nn.Conv2d(10, 1, 1).cuda()
+    inp = torch.rand([1, 1, 20, 20], device="cuda")
+    gen_opt = hvd.DistributedOptimizer(torch.optim.SGD(gen.parameters(), lr=0.1), named_parameters=gen.named_parameters())
+    disc_opt = hvd.DistributedOptimizer(torch.optim.SGD(disc.parameters(), lr=0.1), named_parameters=disc.named_parameters())
+
+    def train_step(train_generator=False, train_discriminator=False):
+        for p in gen.parameters():
+            p.requires_grad_(train_generator)
+        for p in disc.parameters():
+            p.requires_grad_(train_discriminator)
+        gen_opt.zero_grad()
+        disc_opt.zero_grad()
+        disc(gen(inp)).sum().backward()
+        for p in gen.parameters():
+            assert train_generator == (p.grad is not None and bool(p.grad.abs().max() != 0))
+        for p in disc.parameters():
+            assert train_discriminator == (p.grad is not None and bool(p.grad.abs().max() != 0))
+        if train_generator:
+            gen_opt.step()
+        if train_discriminator:
+            disc_opt.step()
+
+    for _ in range(3):
+        train_step(train_generator=True)
+        train_step(train_discriminator=True)
+
+
+def test_gradient_clipping_between_synchronize_and_step(hvd):
+    """test/parallel/test_torch.py:2011-2041."""
+    hvd.init(size=2)
+    model = torch.nn.Linear(1, 1).cuda()
+    with torch.no_grad():
+        model.weight.fill_(0.5)
+        model.bias.zero_()
+    opt = hvd.DistributedOptimizer(torch.optim.SGD(model.parameters(), lr=0.1), named_parameters=model.named_parameters())
+    x = torch.ones(1, 1, device="cuda")
+    loss = torch.nn.functional.mse_loss(model(x), torch.ones(1, 1, device="cuda"))
+    opt.zero_grad()
+    loss.backward()
+    opt.synchronize()
+    prior = model.weight.grad.item()
+    assert prior == pytest.approx(-1.0)  # d/dw (0.5 - 1)^2 = -1 on both ranks, averaged
+    torch.nn.utils.clip_grad_norm_(model.parameters(), 0.1)
+    clipped = model.weight.grad.item()
+    assert abs(prior) > abs(clipped)
+    with opt.skip_synchronize():
+        opt.step()
+    assert model.weight.item() == pytest.approx(0.5 - 0.1 * clipped)
+
+
+def test_no_named_parameters(hvd):
+    """test/parallel/test_torch.py:2076-2100, 2375-2392: generated names."""
+    hvd.init(size=2)
+    torch.manual_seed(7)
+    model = torch.nn.Sequential(torch.nn.Conv2d(1, 20, 1), torch.nn.Conv2d(20, 1, 1)).cuda()
+    opt = hvd.DistributedOptimizer(torch.optim.SGD(model.parameters(), lr=0.1))
+    want = None
+    for _ in range(2):  # the second pass reuses the names of the first
+        opt.zero_grad()
+        model(torch.ones([1, 1, 30, 30], device="cuda")).sum().backward()
+        local = [p.grad.clone() for p in model.parameters()]
+        opt.synchronize()
+        for p, g in zip(model.parameters(), local):
+            assert torch.equal(p.grad, g)  # equal ranks: the average is the gradient
+        with opt.skip_synchronize():
+            opt.step()
+
+
+def test_joined_rank_contributes_zeros_to_a_fused_response(hvd):
+    """test/parallel/test_torch.py:2126-2192 ("two tensors to test fusion"): a rank that has
+    joined takes part with zero-filled tensors, so the average over all ranks is the sum of
+    the others divided by size()."""
+    size = 3
+
+    def peer(rank, name, tensor):  # rank 2 has joined
+        return torch.zeros_like(tensor) if rank == 2 else torch.ones_like(tensor) * (rank + 1)
+
+    hvd.init(size=size, peer_source=peer)
+    a = torch.ones(5, 3, device="cuda")
+    b = torch.ones(7, device="cuda")
+    ha = hvd.allreduce_async(a, name="join.a")
+    hb = hvd.allreduce_async(b, name="join.b")
+    ra, rb = hvd.synchronize(ha), hvd.synchronize(hb)
+    assert torch.allclose(ra, torch.full_like(a, (1 + 2 + 0) / 3))
+    assert torch.allclose(rb, torch.full_like(b, (1 + 2 + 0) / 3))
