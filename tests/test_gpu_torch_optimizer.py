@@ -333,3 +333,33 @@ def test_joined_rank_contributes_zeros_to_a_fused_response(hvd):
     ra, rb = hvd.synchronize(ha), hvd.synchronize(hb)
     assert torch.allclose(ra, torch.full_like(a, (1 + 2 + 0) / 3))
     assert torch.allclose(rb, torch.full_like(b, (1 + 2 + 0) / 3))
+
+
+@pytest.mark.parametrize("opt_cls,kwargs", [(torch.optim.SGD, dict(lr=0.05, momentum=0.9)), (torch.optim.Adam, dict(lr=0.01))])
+@pytest.mark.parametrize("compression", ["none", "fp16"])
+def test_training_loop_equals_the_single_process_loop(hvd, opt_cls, kwargs, compression):
+    """Twenty steps with every rank holding equal gradients (what the reference's tests create by
+    seeding all ranks alike): the average over a power-of-two world is exact, so the distributed
+    run must follow the plain optimizer bit for bit -- with fp16 compression, the plain optimizer
+    fed gradients rounded to half.  Exercises hook -> fuse -> pack -> reduce -> unpack -> step
+    over many steps with the cached plans and changing values."""
+    hvd.init(size=4)
+    ref_model, model = _model(), _model()
+    ref_opt = opt_cls(ref_model.parameters(), **kwargs)
+    comp = hvd.Compression.fp16 if compression == "fp16" else hvd.Compression.none
+    opt = hvd.DistributedOptimizer(opt_cls(model.parameters(), **kwargs), named_parameters=model.named_parameters(),
+                                   compression=comp)
+    torch.manual_seed(11)
+    for step in range(20):
+        x = torch.randn(16, 20, device="cuda")
+        ref_opt.zero_grad()
+        ref_model(x).pow(2).mean().backward()
+        if compression == "fp16":
+            for p in ref_model.parameters():
+                p.grad = p.grad.half().float()
+        ref_opt.step()
+        opt.zero_grad()
+        model(x).pow(2).mean().backward()
+        opt.step()
+        for (n, p), q in zip(model.named_parameters(), ref_model.parameters()):
+            assert torch.equal(p, q), (step, n)
