@@ -29,6 +29,26 @@ struct Add<half_t> {
   }
 };
 
+// acc += x for one 16-byte vector.
+template <typename T, int VEC>
+__device__ __forceinline__ void accumulate(Arr<T, VEC>& acc, const Arr<T, VEC>& x) {
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) acc.v[j] = Add<T>::f(acc.v[j], x.v[j]);
+}
+// Sixteen wrapping byte sums as four word operations each: the low seven bits of every byte
+// add without a carry into the neighbour, the top bit is the exclusive or of the three
+// inputs (both top bits and the carry out of bit 6).
+template <>
+__device__ __forceinline__ void accumulate<uint8_t, 16>(Arr<uint8_t, 16>& acc, const Arr<uint8_t, 16>& x) {
+  uint32_t a[4], b[4];
+  __builtin_memcpy(a, acc.v, 16);
+  __builtin_memcpy(b, x.v, 16);
+#pragma unroll
+  for (int w = 0; w < 4; ++w)
+    a[w] = ((a[w] & 0x7f7f7f7fu) + (b[w] & 0x7f7f7f7fu)) ^ ((a[w] ^ b[w]) & 0x80808080u);
+  __builtin_memcpy(acc.v, a, 16);
+}
+
 constexpr int kMaxK = 8;  // peers per launch; more are folded in by further launches
 
 template <int K>
@@ -65,9 +85,7 @@ __global__ __launch_bounds__(kWG) void reduce_k(T* resident, Peers<K> peers, uin
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
 #pragma unroll
-      for (int k = 0; k < K; ++k)
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[u].v[j] = Add<T>::f(acc[u].v[j], x[u][k].v[j]);
+      for (int k = 0; k < K; ++k) accumulate<T, VEC>(acc[u], x[u][k]);
       stv<T, VEC>(r + (size_t)(v + u * kWG) * VEC, acc[u]);
     }
   }
@@ -75,9 +93,7 @@ __global__ __launch_bounds__(kWG) void reduce_k(T* resident, Peers<K> peers, uin
     V acc = ldv<T, VEC>(r + (size_t)v * VEC);
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-      const V x = ldv<T, VEC>(in[k] + (size_t)v * VEC);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) acc.v[j] = Add<T>::f(acc.v[j], x.v[j]);
+      accumulate<T, VEC>(acc, ldv<T, VEC>(in[k] + (size_t)v * VEC));
     }
     stv<T, VEC>(r + (size_t)v * VEC, acc);
   }
