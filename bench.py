@@ -230,13 +230,13 @@ def cpu_extras(budget_s=2.5):
     def bert():
         off = 0
         for t, c in zip(ts, counts):
-            L.orc_scale_cast_f32_to_f16(P(t), P(hbuf, 2 * off), c_int64(c), c_double(0.125))
+            L.orc_scale_cast_f32_to_f16_f16c(P(t), P(hbuf, 2 * off), c_int64(c), c_double(0.125))
             off += c
         for p in peers:
             L.orc_float16_sum(P(p), P(hbuf), c_int64(n // 8))
         off = 0
         for o, c in zip(outs, counts):
-            L.orc_scale_cast_f16_to_f32(P(hbuf, 2 * off), P(o), c_int64(c), c_double(1.0))
+            L.orc_scale_cast_f16_to_f32_f16c(P(hbuf, 2 * off), P(o), c_int64(c), c_double(1.0))
             off += c
 
     run("bert_large_fp32_to_fp16_7peers_eighth_chunk", bert, 6 * n + 9 * 2 * (n // 8) + 6 * n)

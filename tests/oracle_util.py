@@ -135,17 +135,20 @@ class Oracle:
         self.lib.orc_scale_half_cuda(_p(h), _p(out), c_int64(h.size), c_double(scale))
         return out
 
-    def scale_cast_f32_to_f16(self, x, scale, cast_first=False):
+    def scale_cast_f32_to_f16(self, x, scale, cast_first=False, f16c=False):
         x = np.ascontiguousarray(x, np.float32)
         out = np.empty(x.shape, np.uint16)
         fn = self.lib.orc_cast_then_scale_f32_to_f16 if cast_first else self.lib.orc_scale_cast_f32_to_f16
+        if f16c:
+            fn = self.lib.orc_scale_cast_f32_to_f16_f16c
         fn(_p(x), _p(out), c_int64(x.size), c_double(scale))
         return out
 
-    def scale_cast_f16_to_f32(self, h, scale):
+    def scale_cast_f16_to_f32(self, h, scale, f16c=False):
         h = np.ascontiguousarray(h, np.uint16)
         out = np.empty(h.shape, np.float32)
-        self.lib.orc_scale_cast_f16_to_f32(_p(h), _p(out), c_int64(h.size), c_double(scale))
+        fn = self.lib.orc_scale_cast_f16_to_f32_f16c if f16c else self.lib.orc_scale_cast_f16_to_f32
+        fn(_p(h), _p(out), c_int64(h.size), c_double(scale))
         return out
 
     # ---- sum ----

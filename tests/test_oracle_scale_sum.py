@@ -123,6 +123,23 @@ def test_postscale_and_widen(orc):
         assert np.array_equal(orc.scale_cast_f16_to_f32(h, f).view(np.uint32), want.view(np.uint32))
 
 
+def test_f16c_casts_for_the_cpu_timing_equal_the_software_casts(orc):
+    """The 8-wide variants that the benchmark times on the CPU give the values of the software
+    versions: random magnitudes from subnormal halves to overflow, every non-NaN half, odd lengths."""
+    rng = np.random.default_rng(9)
+    x = (rng.standard_normal(100003) * np.exp(rng.uniform(-20, 12, 100003))).astype(np.float32)
+    x[:6] = [0.0, -0.0, np.inf, -np.inf, 65504.0, 65520.0]
+    for f in (0.125, 1.0, 1.0 / 3.0, -7.5):
+        for n in (0, 1, 7, 8, 9, x.size):
+            assert np.array_equal(orc.scale_cast_f32_to_f16(x[:n], f, f16c=True), orc.scale_cast_f32_to_f16(x[:n], f))
+    h = np.arange(65536, dtype=np.uint16)
+    h = h[~np.isnan(h.view(np.float16))]
+    for f in (1.0, 0.5, 1.0 / 3.0, 1e4):
+        for n in (5, h.size):
+            assert np.array_equal(orc.scale_cast_f16_to_f32(h[:n], f, f16c=True).view(np.uint32),
+                                  orc.scale_cast_f16_to_f32(h[:n], f).view(np.uint32))
+
+
 @pytest.mark.parametrize("dtype,np_t", [(U8, np.uint8), (I8, np.int8), (U16, np.uint16), (I16, np.int16),
                                         (I32, np.int32), (I64, np.int64)])
 def test_sum_integers_wrap(orc, dtype, np_t):
