@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0
 # FETCH_SIZE and WRITE_SIZE runs of `bench.py --kernel-only`, each scaled by what the same
 # counter reads for a plain 256 MiB copy (`bench.py --calibrate`): FETCH_SIZE x 1.9544,
 # WRITE_SIZE x 1.0000.  The summary with the commands is profiles/pack_kernel_fusion_stress.txt.
-PACK_TRAFFIC_BYTES_MEASURED = 93228594
+PACK_TRAFFIC_BYTES_MEASURED = 93214420
 
 
 # One step of the headline is the fusion stress workload as the baseline configuration states it:
@@ -519,7 +519,10 @@ def main():
 
     counts, host, sets = stress_workload(max(1, args.replicas))
     plans = [FusionPlan(src.ptrs, dst.ptrs, counts, F32) for src, dst in sets]
-    fbs = [torch.empty(plans[0].buffer_len, dtype=torch.uint8, device="cuda") for _ in sets]
+    # One fusion buffer per stream slot, reused by every repetition: Horovod's FusionBufferManager keeps
+    # one per (device, framework, stream slot) for the life of the job (ops/gpu_operations.cc:122-124).
+    # The gradient tensors on either side of it rotate over the replicas.
+    fbs = [torch.empty(plans[0].buffer_len, dtype=torch.uint8, device="cuda") for _ in range(2)]
     plan = plans[0]
     payload = 4 * sum(counts)
     torch.cuda.synchronize()
@@ -527,7 +530,7 @@ def main():
 
     def pack():
         i = turn[0] = (turn[0] + 1) % len(plans)
-        plans[i].pack(fbs[i].data_ptr(), 0.125, stream)
+        plans[i].pack(fbs[0].data_ptr(), 0.125, stream)
 
     if args.streams not in (1, 2):
         print("bench.py alternates over one or two stream slots", file=sys.stderr)
@@ -537,8 +540,8 @@ def main():
     def step():
         for _ in range(REPS):
             i = turn[0] = (turn[0] + 1) % len(plans)
-            plans[i].pack(fbs[i].data_ptr(), 0.125, slots[i % len(slots)])
-            plans[i].unpack(fbs[i].data_ptr(), 1.0, slots[i % len(slots)])
+            plans[i].pack(fbs[i % len(slots)].data_ptr(), 0.125, slots[i % len(slots)])
+            plans[i].unpack(fbs[i % len(slots)].data_ptr(), 1.0, slots[i % len(slots)])
 
     def sync_slots():
         for st in slots:
@@ -557,7 +560,9 @@ def main():
     achieved = 2 * payload / ksec / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": PACK_TRAFFIC_BYTES_MEASURED,
-                "kernel": "xfer_k<Scale<float,float>, pack>", "launch_us": round(ksec * 1e6, 2),
+                "kernel": "xfer_k<Scale<float,float>, pack, write-through stores>", "launch_us": round(ksec * 1e6, 2),
+                "timed": "launched back to back on one stream: tensors of another replica every launch, "
+                         "the stream slot's one fusion buffer as the destination",
                 "algorithmic_bytes_per_launch": 2 * payload, "workgroups": plan.num_chunks}
 
     result = {
@@ -566,8 +571,9 @@ def main():
         "ms_per_step": round(sec * 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "fusion stress: 1,024 fp32 tensors, log-uniform 256..65,536 elements (seed 3), "
-                               "U(-1,1) (seed 4); pack with prescale 0.125 into a 64 MiB fusion buffer, unpack, 200 repetitions; "
-                               "consecutive repetitions alternate over the stream slots, each slot with its own buffers",
+                               "U(-1,1) (seed 4); pack with prescale 0.125 into the fusion buffer, unpack, 200 repetitions; "
+                               "consecutive repetitions alternate over the stream slots, each slot with its own persistent "
+                               "fusion buffer (as FusionBufferManager keeps them); the tensors rotate over the replicas",
                    "tensors": len(counts), "payload_bytes": payload, "buffer_len": plan.buffer_len,
                    "repetitions_per_step": REPS, "algorithmic_bytes_per_step": REPS * 4 * payload,
                    "replicas_rotated": len(plans),
@@ -588,8 +594,8 @@ def main():
             def step_alt():
                 for _ in range(REPS):
                     i = turn[0] = (turn[0] + 1) % len(plans)
-                    plans[i].pack(fbs[i].data_ptr(), 0.125, alt[i % len(alt)])
-                    plans[i].unpack(fbs[i].data_ptr(), 1.0, alt[i % len(alt)])
+                    plans[i].pack(fbs[i % len(alt)].data_ptr(), 0.125, alt[i % len(alt)])
+                    plans[i].unpack(fbs[i % len(alt)].data_ptr(), 1.0, alt[i % len(alt)])
 
             def sync_alt():
                 for st in alt:

@@ -199,7 +199,7 @@ struct Axpby<half_t> {
 // data loads are in flight, which saves the finalize launch between the two passes.  All
 // workgroups of a layer execute the same additions in the same order, so they agree to the
 // bit; the layer's first workgroup also stores the sums and coefficients for readers.
-template <typename T, bool FUSED>
+template <typename T, bool FUSED, bool WT>
 __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ chunks, T* a,
                                                     const T* __restrict__ b,
                                                     const double* __restrict__ coeffs,
@@ -216,6 +216,7 @@ __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ ch
   gptr<T> pa = as_global(a + c.tensor);
   gptr<const T> pb = as_global(b + c.tensor);
   const uint32_t nv = n / VEC;
+  const Window out = store_window<WT>(pa, n * (uint32_t)sizeof(T));
   uint32_t v = threadIdx.x;
   double ca, cb;
   if (FUSED) {
@@ -277,7 +278,7 @@ __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ ch
       for (int u = 0; u < kUnroll; ++u) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) x[u].v[j] = Axpby<T>::f(ca, x[u].v[j], cb, y[u].v[j]);
-        stv<T, VEC>(pa + (size_t)(v + u * kWG) * VEC, x[u]);
+        stw<WT, T, VEC>(out, (v + u * kWG) * 16u, x[u]);
       }
       v += kUnroll * kWG;
     }
@@ -297,7 +298,7 @@ __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ ch
     for (int u = 0; u < kUnroll; ++u) {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) x[u].v[j] = Axpby<T>::f(ca, x[u].v[j], cb, y[u].v[j]);
-      stv<T, VEC>(pa + (size_t)(v + u * kWG) * VEC, x[u]);
+      stw<WT, T, VEC>(out, (v + u * kWG) * 16u, x[u]);
     }
   }
   for (; v < nv; v += kWG) {
@@ -305,7 +306,7 @@ __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ ch
     const V y = ldv<T, VEC>(pb + (size_t)v * VEC);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) x.v[j] = Axpby<T>::f(ca, x.v[j], cb, y.v[j]);
-    stv<T, VEC>(pa + (size_t)v * VEC, x);
+    stw<WT, T, VEC>(out, v * 16u, x);
   }
   const uint32_t t = nv * VEC + threadIdx.x;
   if (t < n) pa[t] = Axpby<T>::f(ca, pa[t], cb, pb[t]);
@@ -340,22 +341,22 @@ int plan_dot_norms(hvdhip_adasum_plan* p, const void* a, const void* b, hipStrea
   if (t.nchunks > 0) {
     switch (p->dtype) {
     case HVDHIP_FLOAT16:
-      hipLaunchKernelGGL((dot_partials_k<half_t>), dim3(t.nchunks), dim3(kWG), 0, s, t.chunks,
+      launch(dot_partials_k<half_t>, t.nchunks, s, t.chunks,
                          static_cast<const half_t*>(a), static_cast<const half_t*>(b), p->partials);
       break;
     case HVDHIP_FLOAT32:
-      hipLaunchKernelGGL((dot_partials_k<float>), dim3(t.nchunks), dim3(kWG), 0, s, t.chunks,
+      launch(dot_partials_k<float>, t.nchunks, s, t.chunks,
                          static_cast<const float*>(a), static_cast<const float*>(b), p->partials);
       break;
     default:
-      hipLaunchKernelGGL((dot_partials_k<double>), dim3(t.nchunks), dim3(kWG), 0, s, t.chunks,
+      launch(dot_partials_k<double>, t.nchunks, s, t.chunks,
                          static_cast<const double*>(a), static_cast<const double*>(b), p->partials);
       break;
     }
     HVDHIP_CHECK_LAUNCH("dot_partials_k");
   }
   if (!finalize) return 0;
-  hipLaunchKernelGGL(finalize_k, dim3((uint32_t)p->nlayers), dim3(kWG), 0, s, p->layers, p->partials,
+  launch(finalize_k, (uint32_t)p->nlayers, s, p->layers, p->partials,
                      p->normdots, p->coeffs, std::sqrt(DBL_MIN));
   HVDHIP_CHECK_LAUNCH("finalize_k");
   return 0;
@@ -365,9 +366,14 @@ template <typename T, bool FUSED>
 void launch_scaled_add(hvdhip_adasum_plan* p, void* a, const void* b, const double* coeffs,
                        double ca, double cb, hipStream_t s) {
   const DevTables& t = p->tables;
-  hipLaunchKernelGGL((scaled_add_k<T, FUSED>), dim3(t.nchunks), dim3(kWG), 0, s, t.chunks,
-                     static_cast<T*>(a), static_cast<const T*>(b), coeffs, ca, cb, p->layers,
-                     p->partials, p->normdots, p->coeffs, std::sqrt(DBL_MIN), (uint32_t)p->nlayers);
+  if (write_through(Stores::kAdasum))
+    launch(scaled_add_k<T, FUSED, true>, t.nchunks, s, t.chunks,
+                       static_cast<T*>(a), static_cast<const T*>(b), coeffs, ca, cb, p->layers,
+                       p->partials, p->normdots, p->coeffs, std::sqrt(DBL_MIN), (uint32_t)p->nlayers);
+  else
+    launch(scaled_add_k<T, FUSED, false>, t.nchunks, s, t.chunks,
+                       static_cast<T*>(a), static_cast<const T*>(b), coeffs, ca, cb, p->layers,
+                       p->partials, p->normdots, p->coeffs, std::sqrt(DBL_MIN), (uint32_t)p->nlayers);
 }
 
 template <bool FUSED>

@@ -112,6 +112,16 @@ uint32_t xcd_run(uint64_t nchunks) {
   return nchunks <= kXcdLongRunFrom ? kXcdRun : kXcdLongRun;
 }
 
+bool write_through(Stores family) {
+  constexpr unsigned kDefaultMask = 1u << (unsigned)Stores::kPack | 1u << (unsigned)Stores::kPackNarrowing |
+                                    1u << (unsigned)Stores::kReduceFew | 1u << (unsigned)Stores::kReduceMany;
+  static const unsigned mask = [] {
+    const char* e = std::getenv("HVDHIP_WRITE_THROUGH");
+    return e ? (unsigned)std::strtoul(e, nullptr, 0) : kDefaultMask;
+  }();
+  return (mask >> (unsigned)family) & 1u;
+}
+
 uint32_t xcd_shift(uint64_t nblocks) {
   const uint32_t run = xcd_run(nblocks);
   if (run == 0 || (run & (run - 1)) != 0) return kNoXcdOrder;

@@ -120,6 +120,39 @@ __device__ inline uint32_t xcd_tile(uint32_t block, uint32_t nblocks, uint32_t s
   return block - w + ((w & (kXcds - 1)) << shift) + (w >> 3);
 }
 
+// Launches a streaming kernel: workgroups of kWG lanes, no dynamic LDS.
+template <typename... KArgs, typename... Args>
+inline void launch(void (*kernel)(KArgs...), uint32_t workgroups, hipStream_t stream, Args... args) {
+  hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(kWG), 0, stream, KArgs(args)...);
+}
+
+// Store policy per kernel family: true = write-through buffer stores, false = non-temporal
+// global stores (vecmem.h).  Lines written through are installed in the 256 MB Infinity Cache on
+// their way to HBM, so a kernel that runs next on the same stream and reads them (the collective
+// or reduce-sum after a pack, the unpack after a reduce-sum) finds them there; non-temporal stores
+// bypass it.  Installing costs the writer something (a stress-workload pack launched back to back
+// with nothing reading its output: 18.0 instead of 16.3 us) and saves the reader more (the unpack
+// behind it: 12 instead of 16.4 us), so the kernels whose output the next kernel reads write
+// through, and the ones whose output leaves the pipeline (unpack, batched copies, Adasum's scaled
+// add, a whole-buffer scale) do not.  Measured per family on the pipelines of bench.py, each bit on
+// its own against all off: pack +3 % (two stream slots) to +9 % (one) on the stress workload,
+// +5-7 % on ResNet-50 and GPT-2 XL; narrowing pack +5-8 % on BERT-large; reduce-sum of one peer
+// +6-7 % on ResNet-50 and GPT-2 XL, of seven peers +1 %; unpack 0 to -2 %, widening unpack -4 to
+// -7 %, batched copies -16 %, scaled add -14 %, whole-buffer scale +-0.
+// HVDHIP_WRITE_THROUGH=<mask> (bit = enumerator value) overrides the built-in table, for tuning.
+enum class Stores {
+  kPack = 0,        // same-width pack into the fusion buffer
+  kUnpack = 1,      // same-width unpack out of it
+  kDirect = 2,      // tensor to tensor (batched copies, allgather)
+  kPackNarrowing = 3,   // fp32 -> fp16 pack
+  kUnpackWidening = 4,  // fp16 -> fp32 unpack
+  kContig = 5,      // whole-buffer scale
+  kReduceFew = 6,   // reduce-sum of one or two peers
+  kReduceMany = 7,  // reduce-sum of three to eight peers
+  kAdasum = 8,      // scaled add
+};
+bool write_through(Stores family);
+
 // One contiguous run of elements to transfer (host side only).  `tensor` and
 // `output` are absolute device addresses; `off` is a byte offset into the
 // fusion buffer whose base address is given at launch.  `n` counts elements.

@@ -59,7 +59,7 @@ struct Peers {
 constexpr int kUnroll = 2;
 
 // Workgroup b accumulates K peers into tile t = xcd_tile(b), elements [t*tile, (t+1)*tile).
-template <typename T, int K>
+template <typename T, int K, bool WT>
 __global__ __launch_bounds__(kWG) void reduce_k(T* resident, Peers<K> peers, uint64_t n,
                                                 uint32_t tile, uint32_t run) {
   constexpr int VEC = 16 / (int)sizeof(T);
@@ -72,6 +72,7 @@ __global__ __launch_bounds__(kWG) void reduce_k(T* resident, Peers<K> peers, uin
 #pragma unroll
   for (int k = 0; k < K; ++k) in[k] = as_global(static_cast<const T*>(peers.p[k]) + start);
   const uint32_t nv = m / VEC;
+  const Window out = store_window<WT>(r, m * (uint32_t)sizeof(T));
   uint32_t v = threadIdx.x;
   for (; v + (kUnroll - 1) * kWG < nv; v += kUnroll * kWG) {
     V acc[kUnroll];
@@ -86,7 +87,7 @@ __global__ __launch_bounds__(kWG) void reduce_k(T* resident, Peers<K> peers, uin
     for (int u = 0; u < kUnroll; ++u) {
 #pragma unroll
       for (int k = 0; k < K; ++k) accumulate<T, VEC>(acc[u], x[u][k]);
-      stv<T, VEC>(r + (size_t)(v + u * kWG) * VEC, acc[u]);
+      stw<WT, T, VEC>(out, (v + u * kWG) * 16u, acc[u]);
     }
   }
   for (; v < nv; v += kWG) {
@@ -95,7 +96,7 @@ __global__ __launch_bounds__(kWG) void reduce_k(T* resident, Peers<K> peers, uin
     for (int k = 0; k < K; ++k) {
       accumulate<T, VEC>(acc, ldv<T, VEC>(in[k] + (size_t)v * VEC));
     }
-    stv<T, VEC>(r + (size_t)v * VEC, acc);
+    stw<WT, T, VEC>(out, v * 16u, acc);
   }
   const uint32_t t = nv * VEC + threadIdx.x;
   if (t < m) {
@@ -115,8 +116,12 @@ int launch_k(void* resident, const void* const* incoming, int64_t n, hipStream_t
     const uint32_t blocks = (uint32_t)((slice + tile - 1) / tile);
     Peers<K> peers;
     for (int k = 0; k < K; ++k) peers.p[k] = static_cast<const T*>(incoming[k]) + done;
-    hipLaunchKernelGGL((reduce_k<T, K>), dim3(blocks), dim3(kWG), 0, stream, static_cast<T*>(resident) + done,
-                       peers, slice, tile, xcd_shift(blocks));
+    if (write_through(K <= 2 ? Stores::kReduceFew : Stores::kReduceMany))
+      launch(reduce_k<T, K, true>, blocks, stream, static_cast<T*>(resident) + done,
+                         peers, slice, tile, xcd_shift(blocks));
+    else
+      launch(reduce_k<T, K, false>, blocks, stream, static_cast<T*>(resident) + done,
+                         peers, slice, tile, xcd_shift(blocks));
     HVDHIP_CHECK_LAUNCH("reduce_k");
     done += slice;
     left -= slice;

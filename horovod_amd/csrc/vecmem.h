@@ -89,6 +89,50 @@ __device__ __forceinline__ void stv(gptr<T> p, const Arr<T, N>& a) {
 #endif
 }
 
+// A window over a workgroup's destination range, for stores with a choice of cache policy.
+// WT = false: non-temporal global stores (the lines stay in L2 until they are written back).
+// WT = true: raw buffer stores with the sc0 and sc1 bits, which write the lines through.  Which
+// of the two streams faster depends on the kernel and on what runs around it (measured per
+// kernel family; the table is in context.cc).  A buffer instruction takes its cache policy as an
+// immediate, which is why the write-through path uses one; the window's base must be uniform
+// over the wavefront (the resource lives in scalar registers), and stores beyond `bytes` are
+// dropped by the hardware's range check.
+struct Window {
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint64_t base;
+};
+
+template <bool WT, typename T>
+__device__ __forceinline__ Window store_window(gptr<T> base, uint32_t bytes) {
+  Window w;
+  w.base = reinterpret_cast<uint64_t>(base);
+  if constexpr (WT) {
+    // word 3: 32-bit data format, raw (unstrided, untyped) addressing
+    w.rsrc = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(w.base), 0, (int)bytes, 0x00020000);
+  }
+  return w;
+}
+
+// Stores N elements of T at byte offset `off` of the window.
+template <bool WT, typename T, int N>
+__device__ __forceinline__ void stw(const Window& w, uint32_t off, const Arr<T, N>& a) {
+  if constexpr (WT) {
+#ifndef HVDHIP_WT_AUX
+#define HVDHIP_WT_AUX (1 | 16)  // sc0 | sc1
+#endif
+    constexpr int kScopeBits = HVDHIP_WT_AUX;
+    typedef typename RawSel<(int)sizeof(T) * N>::type R;
+    const R r = __builtin_bit_cast(R, a);
+    if constexpr (sizeof(T) * N == 16) {
+      __builtin_amdgcn_raw_buffer_store_b128(r, w.rsrc, (int)off, 0, kScopeBits);
+    } else {
+      __builtin_amdgcn_raw_buffer_store_b64(r, w.rsrc, (int)off, 0, kScopeBits);
+    }
+  } else {
+    stv<T, N>(reinterpret_cast<gptr<T>>(w.base + off), a);
+  }
+}
+
 }  // namespace hvdhip
 
 #endif  // HVDHIP_VECMEM_H

@@ -129,7 +129,7 @@ struct UnpackF16F32 {
 constexpr int kUnroll = HVDHIP_XFER_UNROLL;  // 16-byte loads in flight per lane
 
 // Streams n elements from src to dst through Op::f with the whole workgroup.
-template <class Op>
+template <class Op, bool WT>
 __device__ __forceinline__ void stream_range(gptr<const typename Op::S> src,
                                              gptr<typename Op::D> dst, uint32_t n,
                                              typename Op::P p) {
@@ -140,6 +140,7 @@ __device__ __forceinline__ void stream_range(gptr<const typename Op::S> src,
   // of an iteration's vectors before it stores any, and touches no address
   // another lane touches.
   const uint32_t nv = n / VEC;
+  const Window out = store_window<WT>(dst, n * (uint32_t)sizeof(D));
   uint32_t v = threadIdx.x;
   for (; v + (kUnroll - 1) * kWG < nv; v += kUnroll * kWG) {
     Arr<S, VEC> x[kUnroll];
@@ -150,7 +151,7 @@ __device__ __forceinline__ void stream_range(gptr<const typename Op::S> src,
       Arr<D, VEC> y;
 #pragma unroll
       for (int j = 0; j < VEC; ++j) y.v[j] = Op::f(x[u].v[j], p);
-      stv<D, VEC>(dst + (size_t)(v + u * kWG) * VEC, y);
+      stw<WT, D, VEC>(out, (v + u * kWG) * (uint32_t)(VEC * sizeof(D)), y);
     }
   }
   for (; v < nv; v += kWG) {
@@ -158,7 +159,7 @@ __device__ __forceinline__ void stream_range(gptr<const typename Op::S> src,
     Arr<D, VEC> y;
 #pragma unroll
     for (int j = 0; j < VEC; ++j) y.v[j] = Op::f(x.v[j], p);
-    stv<D, VEC>(dst + (size_t)v * VEC, y);
+    stw<WT, D, VEC>(out, v * (uint32_t)(VEC * sizeof(D)), y);
   }
   const uint32_t t = nv * VEC + threadIdx.x;  // fewer than VEC elements remain
   if (t < n) dst[t] = Op::f(src[t], p);
@@ -170,7 +171,7 @@ enum Mode { kPack = 0, kUnpack = 1, kDirect = 2 };
 //   kPack:   src = chunk.tensor,      dst = base + chunk.off (pad bytes zeroed)
 //   kUnpack: src = base + chunk.off,  dst = chunk.output
 //   kDirect: src = chunk.tensor,      dst = chunk.output
-template <class Op, int MODE>
+template <class Op, int MODE, bool WT>
 __global__ __launch_bounds__(kWG) void xfer_k(const Chunk* __restrict__ chunks, uint64_t base,
                                               typename Op::P p) {
   typedef typename Op::S S;
@@ -178,20 +179,20 @@ __global__ __launch_bounds__(kWG) void xfer_k(const Chunk* __restrict__ chunks, 
   const Chunk c = chunks[blockIdx.x];
   const uint64_t src_addr = (MODE == kUnpack) ? base + c.off : c.tensor;
   const uint64_t dst_addr = (MODE == kPack) ? base + c.off : c.output;
-  stream_range<Op>(as_global<const S>(src_addr), as_global<D>(dst_addr), c.n, p);
+  stream_range<Op, WT>(as_global<const S>(src_addr), as_global<D>(dst_addr), c.n, p);
   if (MODE == kPack && threadIdx.x < c.pad)
     as_global<uint8_t>(dst_addr)[(uint64_t)c.n * sizeof(D) + threadIdx.x] = 0;
 }
 
 // Contiguous buffer: workgroup b handles tile t = xcd_tile(b), elements [t*tile, (t+1)*tile).
-template <class Op>
+template <class Op, bool WT>
 __global__ __launch_bounds__(kWG) void contig_k(const typename Op::S* src,
                                                 typename Op::D* dst, uint64_t n,
                                                 uint32_t tile, uint32_t run, typename Op::P p) {
   const uint64_t start = (uint64_t)xcd_tile(blockIdx.x, gridDim.x, run) * tile;
   const uint64_t left = n - start;
   const uint32_t m = left < tile ? (uint32_t)left : tile;
-  stream_range<Op>(as_global(src + start), as_global(dst + start), m, p);
+  stream_range<Op, WT>(as_global(src + start), as_global(dst + start), m, p);
 }
 
 // ----------------------------------------------------------------------
@@ -201,7 +202,14 @@ __global__ __launch_bounds__(kWG) void contig_k(const typename Op::S* src,
 template <class Op, int MODE>
 int launch_xfer(const DevTables& t, uint64_t base, typename Op::P p, hipStream_t stream) {
   if (t.nchunks == 0) return 0;
-  hipLaunchKernelGGL((xfer_k<Op, MODE>), dim3(t.nchunks), dim3(kWG), 0, stream, t.chunks, base, p);
+  constexpr bool converting = sizeof(typename Op::S) != sizeof(typename Op::D);
+  const Stores family = MODE == kDirect ? Stores::kDirect
+                        : MODE == kPack ? (converting ? Stores::kPackNarrowing : Stores::kPack)
+                                        : (converting ? Stores::kUnpackWidening : Stores::kUnpack);
+  if (write_through(family))
+    launch(xfer_k<Op, MODE, true>, t.nchunks, stream, t.chunks, base, p);
+  else
+    launch(xfer_k<Op, MODE, false>, t.nchunks, stream, t.chunks, base, p);
   HVDHIP_CHECK_LAUNCH("xfer_k");
   return 0;
 }
@@ -252,7 +260,10 @@ int launch_contig(const void* in, void* out, int64_t n, typename Op::P p, hipStr
   while (left > 0) {  // one launch unless the buffer needs more than kMaxWorkgroups workgroups
     const uint64_t slice = std::min<uint64_t>(left, kMaxWorkgroups * tile);
     const uint32_t blocks = (uint32_t)((slice + tile - 1) / tile);
-    hipLaunchKernelGGL((contig_k<Op>), dim3(blocks), dim3(kWG), 0, stream, src, dst, slice, tile, xcd_shift(blocks), p);
+    if (write_through(Stores::kContig))
+      launch(contig_k<Op, true>, blocks, stream, src, dst, slice, tile, xcd_shift(blocks), p);
+    else
+      launch(contig_k<Op, false>, blocks, stream, src, dst, slice, tile, xcd_shift(blocks), p);
     HVDHIP_CHECK_LAUNCH("contig_k");
     src += slice;
     dst += slice;

@@ -1,6 +1,13 @@
-"""The kernels' multi-vector (unrolled) inner loops only run when a workgroup's chunk holds
-more than 1,024 vectors; the default 4 KiB chunks never reach them for transfers.  This runs
-the pack / scale / reduce parity tests once more in a child process with 64 KiB chunks."""
+"""Library settings that are read from the environment once per process, exercised in child
+processes.
+
+The kernels' multi-vector (unrolled) inner loops only run when a workgroup's chunk holds more
+than 1,024 vectors; the default 4 KiB chunks never reach them for transfers: the pack / scale /
+reduce parity tests run once more with 64 KiB chunks.
+
+Every streaming kernel exists with write-through buffer stores and with non-temporal global
+stores, and a built-in table picks one per kernel family: the same parity tests run with every
+family forced to the one and to the other."""
 import os
 import subprocess
 import sys
@@ -17,6 +24,18 @@ def test_parity_with_64_kib_chunks(gpu):
     cmd = [sys.executable, "-m", "pytest", "-q", "-x", "-m", "gpu", "--timeout", "300", "--timeout-method", "thread",
            os.path.join(ROOT, "tests", "test_gpu_pack.py"), os.path.join(ROOT, "tests", "test_gpu_scale_reduce.py"),
            os.path.join(ROOT, "tests", "test_gpu_adasum.py"), "-p", "no:cacheprovider"]
+    r = subprocess.run(cmd, cwd=ROOT, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=900)
+    tail = r.stdout.decode(errors="replace")[-3000:]
+    assert r.returncode == 0, tail
+    assert " passed" in tail and "failed" not in tail
+
+
+@pytest.mark.parametrize("mask", ["0", "0x1ff"])
+def test_parity_with_every_kernel_family_on_one_store_policy(gpu, mask):
+    env = dict(os.environ, HVDHIP_WRITE_THROUGH=mask)
+    files = ["test_gpu_pack.py", "test_gpu_scale_reduce.py", "test_gpu_adasum.py", "test_gpu_configs.py"]
+    cmd = [sys.executable, "-m", "pytest", "-q", "-x", "-m", "gpu", "--timeout", "300", "--timeout-method", "thread"] + \
+          [os.path.join(ROOT, "tests", f) for f in files] + ["-p", "no:cacheprovider"]
     r = subprocess.run(cmd, cwd=ROOT, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=900)
     tail = r.stdout.decode(errors="replace")[-3000:]
     assert r.returncode == 0, tail
