@@ -276,12 +276,7 @@ class Engine:
         elif first.postscale != 1.0 and nelem:
             H.scale_buffer(result, result, nelem, first.postscale, tdt, s)
 
-        ev = c_void_p()  # completion marker from the event pool
-        check(lib().hvdhip_event_acquire(s.handle, ctypes.byref(ev)), "hvdhip_event_acquire")
-        check(lib().hvdhip_event_record(ev, s.handle), "hvdhip_event_record")
-        marker = Marker(s, ev, len(requests))
-        for r in requests:
-            r.markers.append(marker)
+        self._finish(s, requests)
 
     def _begin(self, group):
         """Picks the stream slot of a fused response and makes it wait for the framework."""
