@@ -78,7 +78,9 @@ __device__ __forceinline__ Triple wg_reduce(Triple t) {
 
 constexpr int kUnroll = 4;
 
-template <typename T>
+// KEEP: the loads leave the vectors in the Infinity Cache for the scaled add that follows
+// (chosen by the host when both vectors fit there with room to spare).
+template <typename T, bool KEEP>
 __global__ __launch_bounds__(kWG) void dot_partials_k(const Chunk* __restrict__ chunks,
                                                       const T* __restrict__ a,
                                                       const T* __restrict__ b,
@@ -96,8 +98,8 @@ __global__ __launch_bounds__(kWG) void dot_partials_k(const Chunk* __restrict__ 
     V x[kUnroll], y[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-      x[u] = ldv<T, VEC>(pa + (size_t)(v + u * kWG) * VEC);
-      y[u] = ldv<T, VEC>(pb + (size_t)(v + u * kWG) * VEC);
+      x[u] = ldv<T, VEC, !KEEP>(pa + (size_t)(v + u * kWG) * VEC);
+      y[u] = ldv<T, VEC, !KEEP>(pb + (size_t)(v + u * kWG) * VEC);
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
@@ -117,7 +119,7 @@ __global__ __launch_bounds__(kWG) void dot_partials_k(const Chunk* __restrict__ 
     }
   }
   for (; v < nv; v += kWG) {
-    const V x = ldv<T, VEC>(pa + (size_t)v * VEC), y = ldv<T, VEC>(pb + (size_t)v * VEC);
+    const V x = ldv<T, VEC, !KEEP>(pa + (size_t)v * VEC), y = ldv<T, VEC, !KEEP>(pb + (size_t)v * VEC);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
       const double p = (double)x.v[j], q = (double)y.v[j];
@@ -333,26 +335,48 @@ struct hvdhip_adasum_plan {
 
 namespace {
 
+// The scaled add reads both vectors a second time.  When the pair is small enough to still be in
+// the 256 MB Infinity Cache by then, the first pass loads it without the non-temporal hint so
+// that it is kept: measured on the combine, +28 % at 2 x 16 MiB, +10 % at 2 x 32 MiB,
+// +6 % at 2 x 64 MiB and +2.5 % at 2 x 128 MiB; at 2 x 256 MiB it costs 0.8 % and beyond that nothing is left of it.
+// HVDHIP_ADASUM_KEEP_BYTES overrides the largest pair (both vectors, bytes) that is kept.
+uint64_t keep_cached_bytes() {
+  static const uint64_t limit = [] {
+    const char* e = std::getenv("HVDHIP_ADASUM_KEEP_BYTES");
+    return e ? (uint64_t)std::strtoull(e, nullptr, 0) : (uint64_t)320 << 20;
+  }();
+  return limit;
+}
+
+template <bool KEEP>
+void launch_dot_partials(hvdhip_adasum_plan* p, const void* a, const void* b, hipStream_t s) {
+  const DevTables& t = p->tables;
+  switch (p->dtype) {
+  case HVDHIP_FLOAT16:
+    launch(dot_partials_k<half_t, KEEP>, t.nchunks, s, t.chunks, static_cast<const half_t*>(a),
+           static_cast<const half_t*>(b), p->partials);
+    break;
+  case HVDHIP_FLOAT32:
+    launch(dot_partials_k<float, KEEP>, t.nchunks, s, t.chunks, static_cast<const float*>(a),
+           static_cast<const float*>(b), p->partials);
+    break;
+  default:
+    launch(dot_partials_k<double, KEEP>, t.nchunks, s, t.chunks, static_cast<const double*>(a),
+           static_cast<const double*>(b), p->partials);
+    break;
+  }
+}
+
 // finalize = false leaves the partial triples for a fused scaled add to sum.
 int plan_dot_norms(hvdhip_adasum_plan* p, const void* a, const void* b, hipStream_t s,
                    bool finalize = true) {
   if (p->nlayers == 0) return 0;
   const DevTables& t = p->tables;
   if (t.nchunks > 0) {
-    switch (p->dtype) {
-    case HVDHIP_FLOAT16:
-      launch(dot_partials_k<half_t>, t.nchunks, s, t.chunks,
-                         static_cast<const half_t*>(a), static_cast<const half_t*>(b), p->partials);
-      break;
-    case HVDHIP_FLOAT32:
-      launch(dot_partials_k<float>, t.nchunks, s, t.chunks,
-                         static_cast<const float*>(a), static_cast<const float*>(b), p->partials);
-      break;
-    default:
-      launch(dot_partials_k<double>, t.nchunks, s, t.chunks,
-                         static_cast<const double*>(a), static_cast<const double*>(b), p->partials);
-      break;
-    }
+    if (2 * (uint64_t)p->total * (uint64_t)dtype_size(p->dtype) <= keep_cached_bytes())
+      launch_dot_partials<true>(p, a, b, s);
+    else
+      launch_dot_partials<false>(p, a, b, s);
     HVDHIP_CHECK_LAUNCH("dot_partials_k");
   }
   if (!finalize) return 0;
@@ -490,7 +514,8 @@ int hvdhip_adasum_plan_create(const int* tensor_counts, int nlayers, int dtype,
   (void)hipGetDevice(&p->device);
   {
     std::vector<Chunk> ordered(chunks.size());
-    for (size_t c = 0; c < chunks.size(); ++c) ordered[xcd_slot(c, chunks.size(), xcd_run(chunks.size()))] = chunks[c];
+    const uint32_t run = xcd_run(chunks.size(), chunk_bytes(Family::kAdasum), true);
+    for (size_t c = 0; c < chunks.size(); ++c) ordered[xcd_slot(c, chunks.size(), run)] = chunks[c];
     chunks.swap(ordered);
   }
   int rc = upload_chunks(chunks, &p->tables);

@@ -103,13 +103,16 @@ uint64_t count_chunks(const std::vector<Seg>& segs, uint32_t chunk_units) {
   return nchunks > kMaxWorkgroups ? ~0ull : nchunks;
 }
 
-uint32_t xcd_run(uint64_t nchunks) {
+uint32_t xcd_run(uint64_t nchunks, uint32_t chunk_bytes, bool long_runs) {
   static const long forced = [] {
     const char* e = std::getenv("HVDHIP_XCD_RUN");
     return e ? std::strtol(e, nullptr, 10) : -1L;
   }();
   if (forced >= 0) return (uint32_t)forced;
-  return nchunks <= kXcdLongRunFrom ? kXcdRun : kXcdLongRun;
+  if (chunk_bytes == 0) return 0;
+  const uint32_t bytes =
+      !long_runs && nchunks * (uint64_t)chunk_bytes <= kXcdLongRunFrom ? kXcdRunBytes : kXcdLongRunBytes;
+  return bytes > chunk_bytes ? bytes / chunk_bytes : 1;
 }
 
 bool write_through(Stores family) {
@@ -122,8 +125,8 @@ bool write_through(Stores family) {
   return (mask >> (unsigned)family) & 1u;
 }
 
-uint32_t xcd_shift(uint64_t nblocks) {
-  const uint32_t run = xcd_run(nblocks);
+uint32_t xcd_shift(uint64_t nblocks, uint32_t tile_bytes) {
+  const uint32_t run = xcd_run(nblocks, tile_bytes);
   if (run == 0 || (run & (run - 1)) != 0) return kNoXcdOrder;
   uint32_t shift = 0;
   while ((1u << shift) < run) ++shift;
@@ -132,7 +135,7 @@ uint32_t xcd_shift(uint64_t nblocks) {
 
 void fill_chunks(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t tensor_es,
                  uint32_t buffer_es, Chunk* out, uint64_t nchunks) {
-  const uint32_t run = xcd_run(nchunks);
+  const uint32_t run = xcd_run(nchunks, chunk_units * (tensor_es > buffer_es ? tensor_es : buffer_es));
   uint64_t index = 0;
   for (const Seg& s : segs) {
     const uint64_t nbytes = s.n * buffer_es;

@@ -83,16 +83,20 @@ uint32_t chunk_bytes(Family f);
 // (1.5-2.5 % on the pack and unpack kernels, up to 5 % on the widening unpack) when one XCD walks
 // runs of consecutive chunks instead of every eighth chunk, so tables and tile numbers are laid out
 // accordingly: within each group of 8 * run chunks, XCD x gets chunks x * run .. x * run + run - 1.
-// The ragged end (fewer than 8 * run chunks) keeps its natural order.  Measured against natural
-// order: runs of 64 chunks are best for launches of 16-128 MiB (+2-5 % on every kernel family; 32-256
-// are close, 1 and >= 1,024 gain nothing) but cost 2-6 % at 512 MiB and more, where runs of 256 gain
-// 1-3 %; so launches of more than kXcdLongRunFrom chunks use the longer run.  HVDHIP_XCD_RUN
-// overrides the run length for every launch, 0 switches the reordering off.
+// The ragged end (fewer than 8 * run chunks) keeps its natural order.  What counts is the length of
+// a run in bytes.  Measured against natural order: 256 KiB per run is best for launches of 16-128
+// MiB (+2-5 % on every kernel family; 128 KiB - 1 MiB are close, a single chunk and >= 4 MiB gain
+// nothing) but costs 2-6 % at 512 MiB and more, where 1 MiB gains 1-3 % and 4 MiB loses 4-6 %; so
+// launches that cover more than kXcdLongRunFrom bytes use the longer run.  HVDHIP_XCD_RUN overrides
+// the run length (in chunks) for every launch, 0 switches the reordering off.
 constexpr uint32_t kXcds = 8;
-constexpr uint32_t kXcdRun = 64;
-constexpr uint32_t kXcdLongRun = 256;
-constexpr uint64_t kXcdLongRunFrom = 32768;  // 128 MiB of 4 KiB chunks
-uint32_t xcd_run(uint64_t nchunks);
+constexpr uint32_t kXcdRunBytes = 256u << 10;
+constexpr uint32_t kXcdLongRunBytes = 1u << 20;
+constexpr uint64_t kXcdLongRunFrom = 128ull << 20;
+// Run length in chunks for a launch of nchunks chunks of chunk_bytes each (at least one chunk).
+// The Adasum kernels (two read streams of 16 KiB chunks) do best with the longer run at every size
+// (2 x 16 MiB: 13.9 against 14.2 us, 2 x 64 MiB: 53.0 against 54.2 us): long_runs asks for it.
+uint32_t xcd_run(uint64_t nchunks, uint32_t chunk_bytes, bool long_runs = false);
 // Chunk (or tile) that the workgroup at table position `slot` handles.
 __host__ __device__ inline uint64_t xcd_chunk(uint64_t slot, uint64_t nchunks, uint32_t run) {
   const uint64_t group = (uint64_t)kXcds * run;
@@ -111,7 +115,7 @@ __host__ __device__ inline uint64_t xcd_slot(uint64_t chunk, uint64_t nchunks, u
 // The same mapping for kernels that number their tiles themselves, in shifts and masks: shift =
 // log2(run) for a power-of-two run, kNoXcdOrder for workgroup order = tile order.
 constexpr uint32_t kNoXcdOrder = 32;
-uint32_t xcd_shift(uint64_t nblocks);
+uint32_t xcd_shift(uint64_t nblocks, uint32_t tile_bytes);
 __device__ inline uint32_t xcd_tile(uint32_t block, uint32_t nblocks, uint32_t shift) {
   if (shift >= kNoXcdOrder) return block;
   const uint32_t mask = (kXcds << shift) - 1;  // group of 8 * run tiles

@@ -118,10 +118,10 @@ int launch_k(void* resident, const void* const* incoming, int64_t n, hipStream_t
     for (int k = 0; k < K; ++k) peers.p[k] = static_cast<const T*>(incoming[k]) + done;
     if (write_through(K <= 2 ? Stores::kReduceFew : Stores::kReduceMany))
       launch(reduce_k<T, K, true>, blocks, stream, static_cast<T*>(resident) + done,
-                         peers, slice, tile, xcd_shift(blocks));
+                         peers, slice, tile, xcd_shift(blocks, tile * (uint32_t)sizeof(T)));
     else
       launch(reduce_k<T, K, false>, blocks, stream, static_cast<T*>(resident) + done,
-                         peers, slice, tile, xcd_shift(blocks));
+                         peers, slice, tile, xcd_shift(blocks, tile * (uint32_t)sizeof(T)));
     HVDHIP_CHECK_LAUNCH("reduce_k");
     done += slice;
     left -= slice;

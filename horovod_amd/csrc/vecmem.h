@@ -66,15 +66,17 @@ struct Arr {
 #define HVDHIP_NONTEMPORAL 1
 #endif
 
-template <typename T, int N>
+// NT = false loads without the hint, for data that a later kernel reads again while it can
+// still be in the Infinity Cache.
+template <typename T, int N, bool NT = true>
 __device__ __forceinline__ Arr<T, N> ldv(gptr<const T> p) {
   typedef typename Raw<(int)sizeof(T) * N, (int)alignof(T)>::type R;
-#if HVDHIP_NONTEMPORAL
-  const typename RawSel<(int)sizeof(T) * N>::type r =
-      __builtin_nontemporal_load(reinterpret_cast<gptr<const R>>(p));
-#else
-  const typename RawSel<(int)sizeof(T) * N>::type r = *reinterpret_cast<gptr<const R>>(p);
-#endif
+  typename RawSel<(int)sizeof(T) * N>::type r;
+  if constexpr (NT && HVDHIP_NONTEMPORAL) {
+    r = __builtin_nontemporal_load(reinterpret_cast<gptr<const R>>(p));
+  } else {
+    r = *reinterpret_cast<gptr<const R>>(p);
+  }
   return __builtin_bit_cast(Arr<T, N>, r);
 }
 

@@ -261,9 +261,9 @@ int launch_contig(const void* in, void* out, int64_t n, typename Op::P p, hipStr
     const uint64_t slice = std::min<uint64_t>(left, kMaxWorkgroups * tile);
     const uint32_t blocks = (uint32_t)((slice + tile - 1) / tile);
     if (write_through(Stores::kContig))
-      launch(contig_k<Op, true>, blocks, stream, src, dst, slice, tile, xcd_shift(blocks), p);
+      launch(contig_k<Op, true>, blocks, stream, src, dst, slice, tile, xcd_shift(blocks, chunk_bytes(Family::kXfer)), p);
     else
-      launch(contig_k<Op, false>, blocks, stream, src, dst, slice, tile, xcd_shift(blocks), p);
+      launch(contig_k<Op, false>, blocks, stream, src, dst, slice, tile, xcd_shift(blocks, chunk_bytes(Family::kXfer)), p);
     HVDHIP_CHECK_LAUNCH("contig_k");
     src += slice;
     dst += slice;
