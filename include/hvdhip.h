@@ -232,7 +232,11 @@ int64_t hvdhip_fusion_plan_num_chunks(const hvdhip_fusion_plan* plan);
  * every tensor to its offset, multiplying by scale_factor and, for a
  * converting plan, rounding fp32 to fp16 (nearest even).  Pad bytes between
  * entries are written as zero so that a reduction over the whole padded
- * buffer reads defined values. */
+ * buffer reads defined values.  The buffer is written through the device's
+ * 256 MB Infinity Cache, where the next kernel or collective on the stream
+ * finds it; pass the same buffer for a stream slot every time (the
+ * reference keeps one per slot, ops/gpu_operations.cc:122-124), which is
+ * also the fastest for this call. */
 int hvdhip_fusion_pack(hvdhip_fusion_plan* plan, void* fusion_buffer, double scale_factor,
                        unsigned flags, void* stream);
 
