@@ -446,6 +446,12 @@ void AdasumGPU::FusedPairwiseReduce(void* a, const void* b, DataType horovod_dat
   hvdhip_adasum_plan* plan;
   auto it = plans_.find(key);
   if (it == plans_.end()) {
+    if (plans_.size() >= kMaxAdasumPlans) {
+      // layer layouts repeat from step to step; a caller that keeps producing new ones starts over
+      // (destroying a plan waits for the device, so nothing queued can still use it)
+      for (auto& kv : plans_) hvdhip_adasum_plan_destroy(kv.second);
+      plans_.clear();
+    }
     plan = nullptr;
     gpu_context_->ErrorCheck("hvdhip_adasum_plan_create",
                              hvdhip_adasum_plan_create(tensor_counts.data(), (int)tensor_counts.size(),

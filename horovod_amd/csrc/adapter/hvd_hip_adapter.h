@@ -225,6 +225,7 @@ public:
 
 private:
   GPUContext* gpu_context_;
+  static constexpr size_t kMaxAdasumPlans = 128;
   std::map<std::pair<std::pair<int, const void*>, std::vector<int>>, hvdhip_adasum_plan*> plans_;  // (dtype, stream), counts
 };
 
