@@ -6,7 +6,9 @@
 // device-resident table of self-contained 32-byte chunk entries (source,
 // destination, fusion-buffer offset, element count), one per workgroup.  A
 // workgroup of four wave64 wavefronts loads its entry with a single scalar
-// load and streams its chunk with one 16-byte non-temporal access per lane
+// load and streams its chunk with one 16-byte access per lane each way: non-temporal
+// loads, and stores that either bypass the Infinity Cache or write through it for
+// the kernel that reads the destination next
 // (4 KiB per workgroup: the occupancy of many small workgroups keeps about
 // 8 MiB in flight, which is what HBM latency times bandwidth asks for).
 // Workgroups are dispatched round-robin over the XCDs and consecutive
