@@ -6,14 +6,14 @@
 // device-resident table of self-contained 32-byte chunk entries (source,
 // destination, fusion-buffer offset, element count), one per workgroup.  A
 // workgroup of four wave64 wavefronts loads its entry with a single scalar
-// load and streams its chunk with one 16-byte access per lane each way: non-temporal
-// loads, and stores that either bypass the Infinity Cache or write through it for
-// the kernel that reads the destination next
+// load and streams its chunk with one 16-byte access per lane each way
 // (4 KiB per workgroup: the occupancy of many small workgroups keeps about
 // 8 MiB in flight, which is what HBM latency times bandwidth asks for).
-// Workgroups are dispatched round-robin over the XCDs and consecutive
-// workgroups touch consecutive 4 KiB pieces, so a single big tensor is spread
-// over all XCDs and HBM stacks while a tiny one costs a single short
+// Loads are non-temporal; stores either bypass the Infinity Cache or write
+// through it for the kernel that reads the destination next.  Workgroups are
+// dispatched round-robin over the XCDs and the table is ordered so that each
+// XCD walks runs of consecutive chunks: a single big tensor is spread over
+// all XCDs and HBM stacks while a tiny one costs a single short
 // workgroup.  This is bandwidth-bound byte/element work with no reuse: no
 // LDS and no matrix cores are involved.
 //
