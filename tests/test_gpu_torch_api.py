@@ -393,3 +393,50 @@ def test_adasum_responses_on_alternating_streams_do_not_share_state(hvd, orc):
         want = orc.adasum_pairwise(_np(t), peer, [t.numel()], F32)[0]
         ulp = np.abs(_np(out).view(np.int32).astype(np.int64) - want.view(np.int32).astype(np.int64))
         assert ulp.max() <= 1, n
+
+
+def _adasum_reference_operation(a, b):
+    """test/parallel/test_adasum_tensorflow.py:28-43, in float64."""
+    anormsq, bnormsq = np.inner(a.ravel(), a.ravel()), np.inner(b.ravel(), b.ravel())
+    dot = np.dot(a.ravel(), b.ravel())
+    acoeff = 1.0 - dot / anormsq * 0.5 if anormsq != 0 else 1.0
+    bcoeff = 1.0 - dot / bnormsq * 0.5 if bnormsq != 0 else 1.0
+    return acoeff * a + bcoeff * b
+
+
+def _reference_tree_reduction(tensors):
+    """test_adasum_tensorflow.py:48-59: neighbours first, then the pairs' results."""
+    level = list(tensors)
+    while len(level) > 1:
+        level = [_adasum_reference_operation(level[2 * i], level[2 * i + 1]) for i in range(len(level) // 2)]
+    return level[0]
+
+
+@pytest.mark.parametrize("size,local_size", [(2, 1), (4, 1), (8, 1), (8, 2), (4, 4)])
+def test_adasum_against_the_reference_tests_numpy_tree(hvd, size, local_size):
+    """test_adasum_tensorflow.py:103-176 (CPU and GPU-NCCL variants): two 2x2 tensors of uniform
+    [0, 1) values per rank, each reduced on its own; expected = the numpy tree over the nodes'
+    sums, divided by local_size; fp16, fp32 and fp64, compared with the tolerances of
+    assertAllCloseAccordingToType (1e-3 for half, 1e-6 otherwise)."""
+    rng = np.random.default_rng(17)
+    rank_tensors = [[rng.random((2, 2)), rng.random((2, 2))] for _ in range(size)]
+    table = {}
+
+    def peer(rank, name, tensor):
+        return table[(rank, name)]
+
+    hvd.init(size=size, local_size=local_size, peer_source=peer)
+    nodes = size // local_size
+    for dtype, tol in [(torch.float16, 1e-3), (torch.float32, 1e-6), (torch.float64, 1e-6)]:
+        for which in range(2):
+            name = "ref.%s.%d" % (str(dtype).split(".")[1], which)
+            cast = [torch.from_numpy(rank_tensors[r][which]).cuda().type(dtype) for r in range(size)]
+            for r in range(1, size):
+                table[(r, "allreduce." + name)] = cast[r]
+            got = hvd.allreduce(cast[0], op=hvd.Adasum, name=name)
+            # the expectation starts from the values as cast, like the tensors the ranks pass
+            held = [c.double().cpu().numpy() for c in cast]
+            sums = [sum(held[n * local_size:(n + 1) * local_size]) for n in range(nodes)]
+            want = _reference_tree_reduction(sums) / local_size
+            assert got.dtype == dtype
+            assert np.allclose(got.double().cpu().numpy(), want, rtol=tol, atol=tol), (dtype, size, local_size)
