@@ -73,15 +73,36 @@ __global__ __launch_bounds__(kWG) void reduce_k(T* resident, Peers<K> peers, uin
   for (int k = 0; k < K; ++k) in[k] = as_global(static_cast<const T*>(peers.p[k]) + start);
   const uint32_t nv = m / VEC;
   const Window out = store_window<WT>(r, m * (uint32_t)sizeof(T));
+  constexpr bool kBytes = sizeof(T) == 1;  // byte elements are read through windows (vecmem.h)
+  ReadWindow rin, pin[K];
+  if constexpr (kBytes) {
+    rin = load_window(gptr<const T>(r), m);
+#pragma unroll
+    for (int k = 0; k < K; ++k) pin[k] = load_window(in[k], m);
+  }
+  auto load_resident = [&](uint32_t vec) {
+    if constexpr (kBytes) {
+      return ldw<T, VEC>(rin, vec * 16u);
+    } else {
+      return ldv<T, VEC>(r + (size_t)vec * VEC);
+    }
+  };
+  auto load_peer = [&](int k, uint32_t vec) {
+    if constexpr (kBytes) {
+      return ldw<T, VEC>(pin[k], vec * 16u);
+    } else {
+      return ldv<T, VEC>(in[k] + (size_t)vec * VEC);
+    }
+  };
   uint32_t v = threadIdx.x;
   for (; v + (kUnroll - 1) * kWG < nv; v += kUnroll * kWG) {
     V acc[kUnroll];
     V x[kUnroll][K];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-      acc[u] = ldv<T, VEC>(r + (size_t)(v + u * kWG) * VEC);
+      acc[u] = load_resident(v + u * kWG);
 #pragma unroll
-      for (int k = 0; k < K; ++k) x[u][k] = ldv<T, VEC>(in[k] + (size_t)(v + u * kWG) * VEC);
+      for (int k = 0; k < K; ++k) x[u][k] = load_peer(k, v + u * kWG);
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
@@ -91,10 +112,10 @@ __global__ __launch_bounds__(kWG) void reduce_k(T* resident, Peers<K> peers, uin
     }
   }
   for (; v < nv; v += kWG) {
-    V acc = ldv<T, VEC>(r + (size_t)v * VEC);
+    V acc = load_resident(v);
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-      accumulate<T, VEC>(acc, ldv<T, VEC>(in[k] + (size_t)v * VEC));
+      accumulate<T, VEC>(acc, load_peer(k, v));
     }
     stw<WT, T, VEC>(out, v * 16u, acc);
   }

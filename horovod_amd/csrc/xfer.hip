@@ -143,11 +143,21 @@ __device__ __forceinline__ void stream_range(gptr<const typename Op::S> src,
   // another lane touches.
   const uint32_t nv = n / VEC;
   const Window out = store_window<WT>(dst, n * (uint32_t)sizeof(D));
+  constexpr bool kBytes = sizeof(S) == 1;  // byte elements are read through a window (vecmem.h)
+  ReadWindow in;
+  if constexpr (kBytes) in = load_window(src, n);
+  auto load = [&](uint32_t vec) {
+    if constexpr (kBytes) {
+      return ldw<S, VEC>(in, vec * 16u);
+    } else {
+      return ldv<S, VEC>(src + (size_t)vec * VEC);
+    }
+  };
   uint32_t v = threadIdx.x;
   for (; v + (kUnroll - 1) * kWG < nv; v += kUnroll * kWG) {
     Arr<S, VEC> x[kUnroll];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) x[u] = ldv<S, VEC>(src + (size_t)(v + u * kWG) * VEC);
+    for (int u = 0; u < kUnroll; ++u) x[u] = load(v + u * kWG);
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       Arr<D, VEC> y;
@@ -157,7 +167,7 @@ __device__ __forceinline__ void stream_range(gptr<const typename Op::S> src,
     }
   }
   for (; v < nv; v += kWG) {
-    const Arr<S, VEC> x = ldv<S, VEC>(src + (size_t)v * VEC);
+    const Arr<S, VEC> x = load(v);
     Arr<D, VEC> y;
 #pragma unroll
     for (int j = 0; j < VEC; ++j) y.v[j] = Op::f(x.v[j], p);
@@ -284,6 +294,10 @@ int launch_contig(const void* in, void* out, int64_t n, typename Op::P p, hipStr
 // asynchronous copy on the caller's stream, and the kernel follows on the
 // same stream.  Evicted entries hand their buffers to the next miss; before
 // that, the entry's last-use event is waited for (normally long complete).
+// That event costs a command on the stream after every launch (about 3 us
+// between two 17 us copies), so it is only recorded while the cache is full
+// and entries are being evicted; a victim whose last use went unrecorded
+// makes the eviction wait for the whole device once.
 
 struct TableBuf {
   void* dev = nullptr;
@@ -295,7 +309,10 @@ struct CachedCopy {
   std::vector<uint64_t> key;  // unit size, n, then out/in/size triples
   DevTables tables;           // tables.alloc is not owned: it aliases buf.dev
   TableBuf buf;
-  hipEvent_t done = nullptr;        // recorded after every launch that reads the table
+  hipEvent_t uploaded = nullptr;    // recorded once, behind the table's upload on the stream that built it
+  bool upload_complete = false;     // `uploaded` has been seen complete: other streams need not wait for it
+  hipEvent_t done = nullptr;        // recorded after a launch that reads the table, while the cache is full
+  bool done_is_latest = false;      // the latest launch was followed by a record of `done`
   hipStream_t last_stream = nullptr;
   bool several_streams = false;     // used on more than one stream since it was built
 };
@@ -357,12 +374,13 @@ int acquire_buf(CopyCache& c, size_t bytes, TableBuf* out) {
 // still read its table, and keeps its buffers for reuse.
 int evict_one(CopyCache& c) {
   CachedCopy& victim = c.lru.back();
-  if (victim.several_streams) {
+  if (victim.several_streams || !victim.done_is_latest) {
     HVDHIP_CHECK(hipDeviceSynchronize());
-  } else if (victim.done) {
+  } else {
     HVDHIP_CHECK(hipEventSynchronize(victim.done));
   }
   if (victim.done) (void)hipEventDestroy(victim.done);
+  if (victim.uploaded) (void)hipEventDestroy(victim.uploaded);
   if (c.spare.size() < kSpareBufs) {
     c.spare.push_back(victim.buf);
   } else {
@@ -391,8 +409,15 @@ int cached_tables(CopyCache& c, void* const* out, const void* const* in, const s
       c.lru.splice(c.lru.begin(), c.lru, it);
       CachedCopy* hit = &c.lru.front();
       // The table was uploaded asynchronously on the stream that built it; another stream
-      // must not read it earlier.  `done` was recorded on that stream after the upload.
-      if (stream != hit->last_stream) HVDHIP_CHECK(hipStreamWaitEvent(stream, hit->done, 0));
+      // must not read it earlier.
+      if (!hit->upload_complete) {
+        if (hipEventQuery(hit->uploaded) == hipSuccess) {
+          hit->upload_complete = true;
+        } else {
+          (void)hipGetLastError();  // hipErrorNotReady is not an error here
+          if (stream != hit->last_stream) HVDHIP_CHECK(hipStreamWaitEvent(stream, hit->uploaded, 0));
+        }
+      }
       *result = hit;
       return 0;
     }
@@ -412,13 +437,16 @@ int cached_tables(CopyCache& c, void* const* out, const void* const* in, const s
   int rc = acquire_buf(c, bytes ? bytes : 32, &entry.buf);
   if (rc) return rc;
   hipError_t e = hipEventCreateWithFlags(&entry.done, hipEventDisableTiming);
+  if (e == hipSuccess) e = hipEventCreateWithFlags(&entry.uploaded, hipEventDisableTiming);
   if (e == hipSuccess && nchunks) {
     fill_chunks(segs, chunk_units, unit, unit, static_cast<Chunk*>(entry.buf.pinned), nchunks);
     e = hipMemcpyAsync(entry.buf.dev, entry.buf.pinned, bytes, hipMemcpyHostToDevice, stream);
   }
+  if (e == hipSuccess) e = hipEventRecord(entry.uploaded, stream);
   if (e != hipSuccess) {
     (void)hipGetLastError();
     if (entry.done) (void)hipEventDestroy(entry.done);
+    if (entry.uploaded) (void)hipEventDestroy(entry.uploaded);
     // the copy may have been queued: do not hand the buffers on before the stream is idle
     (void)hipStreamSynchronize(stream);
     c.spare.push_back(entry.buf);
@@ -434,11 +462,16 @@ int cached_tables(CopyCache& c, void* const* out, const void* const* in, const s
   return 0;
 }
 
-// Records that `stream` now holds work reading the entry's table.
-int mark_used(CachedCopy* entry, hipStream_t stream) {
+// Notes that `stream` now holds work reading the entry's table, with an event behind it while
+// the cache is full (the next miss will evict).
+int mark_used(CopyCache& c, CachedCopy* entry, hipStream_t stream) {
   if (stream != entry->last_stream) entry->several_streams = true;
   entry->last_stream = stream;
-  HVDHIP_CHECK(hipEventRecord(entry->done, stream));
+  entry->done_is_latest = false;
+  if (c.lru.size() >= kCopyCacheCapacity) {
+    HVDHIP_CHECK(hipEventRecord(entry->done, stream));
+    entry->done_is_latest = true;
+  }
   return 0;
 }
 
@@ -484,7 +517,7 @@ int hvdhip_batched_d2d_memcpy(void* const* out, const void* const* in, const siz
   rc = cached_tables(*cache, out, in, sizes, num_copies, 1, s, &entry);
   if (rc) return rc;
   rc = launch_xfer<Copy<uint8_t>, kDirect>(entry->tables, 0, {}, s);
-  int rc2 = mark_used(entry, s);
+  int rc2 = mark_used(*cache, entry, s);
   if (rc == 0) rc = rc2;
   return rc ? rc : ok();
 }
@@ -513,7 +546,7 @@ int hvdhip_batched_scaled_d2d_memcpy(void* const* out, const void* const* in,
   rc = cached_tables(*cache, out, in, sizes, num_copies, es, s, &entry);
   if (rc) return rc;
   rc = launch_same_dtype<kDirect>(entry->tables, 0, scale_factor, dtype, s);
-  int rc2 = mark_used(entry, s);
+  int rc2 = mark_used(*cache, entry, s);
   if (rc == 0) rc = rc2;
   return rc ? rc : ok();
 }
