@@ -3,6 +3,7 @@
 Device memory comes from the caller (torch tensors here, the framework in
 Horovod); these classes only pass raw addresses through.
 """
+import array
 import ctypes
 from ctypes import c_double, c_float, c_int, c_int64, c_size_t, c_void_p
 
@@ -10,10 +11,15 @@ from ._lib import DTYPE, check, lib
 
 
 def _ptr_array(values):
-    arr = (c_void_p * len(values))()
-    for i, v in enumerate(values):
-        arr[i] = v
-    return arr
+    """A C array of addresses; through array.array, which converts a list several times faster
+    than filling a ctypes array element by element."""
+    raw = array.array("Q", values)
+    return (c_void_p * len(raw)).from_buffer(raw) if len(raw) else (c_void_p * 0)()
+
+
+def _size_array(values):
+    raw = array.array("Q", values)
+    return (c_size_t * len(raw)).from_buffer(raw) if len(raw) else (c_size_t * 0)()
 
 
 class Stream:
@@ -136,14 +142,14 @@ class AdasumPlan:
 
 def batched_d2d_memcpy(out_ptrs, in_ptrs, sizes, stream):
     n = len(sizes)
-    check(lib().hvdhip_batched_d2d_memcpy(_ptr_array(out_ptrs), _ptr_array(in_ptrs), (c_size_t * n)(*sizes), n,
+    check(lib().hvdhip_batched_d2d_memcpy(_ptr_array(out_ptrs), _ptr_array(in_ptrs), _size_array(sizes), n,
                                           stream.handle), "hvdhip_batched_d2d_memcpy")
 
 
 def batched_scaled_d2d_memcpy(out_ptrs, in_ptrs, sizes, scale, dtype, stream):
     n = len(sizes)
     check(lib().hvdhip_batched_scaled_d2d_memcpy(_ptr_array(out_ptrs), _ptr_array(in_ptrs),
-                                                 (c_size_t * n)(*sizes), n, float(scale), int(dtype),
+                                                 _size_array(sizes), n, float(scale), int(dtype),
                                                  stream.handle), "hvdhip_batched_scaled_d2d_memcpy")
 
 
