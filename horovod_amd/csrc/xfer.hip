@@ -436,8 +436,10 @@ int cached_tables(CopyCache& c, void* const* out, const void* const* in, const s
   const size_t bytes = (size_t)nchunks * sizeof(Chunk);
   int rc = acquire_buf(c, bytes ? bytes : 32, &entry.buf);
   if (rc) return rc;
-  hipError_t e = hipEventCreateWithFlags(&entry.done, hipEventDisableTiming);
-  if (e == hipSuccess) e = hipEventCreateWithFlags(&entry.uploaded, hipEventDisableTiming);
+  // internal ordering only (table uploads and table reads): no timing, no system-scope fence
+  constexpr unsigned kOrderOnly = hipEventDisableTiming | hipEventDisableSystemFence;
+  hipError_t e = hipEventCreateWithFlags(&entry.done, kOrderOnly);
+  if (e == hipSuccess) e = hipEventCreateWithFlags(&entry.uploaded, kOrderOnly);
   if (e == hipSuccess && nchunks) {
     fill_chunks(segs, chunk_units, unit, unit, static_cast<Chunk*>(entry.buf.pinned), nchunks);
     e = hipMemcpyAsync(entry.buf.dev, entry.buf.pinned, bytes, hipMemcpyHostToDevice, stream);
