@@ -44,9 +44,9 @@ REPS = 200
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10,
+    ap.add_argument("--steps", type=int, default=20,
                     help="timed steps; one step is the workload's %d repetitions of pack + unpack" % REPS)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--kernel-only", nargs="?", const="pack", default=None,
