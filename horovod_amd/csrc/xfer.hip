@@ -296,8 +296,9 @@ int launch_contig(const void* in, void* out, int64_t n, typename Op::P p, hipStr
 // that, the entry's last-use event is waited for (normally long complete).
 // That event costs a command on the stream after every launch (about 3 us
 // between two 17 us copies), so it is only recorded while the cache is full
-// and entries are being evicted; a victim whose last use went unrecorded
-// makes the eviction wait for the whole device once.
+// and entries are being evicted (or were, within the last 256 launches); a
+// victim whose last use went unrecorded makes the eviction wait for the whole
+// device once.
 
 struct TableBuf {
   void* dev = nullptr;
@@ -323,6 +324,12 @@ struct CopyCache {
   std::mutex mu;
   std::list<CachedCopy> lru;  // front = most recent
   std::vector<TableBuf> spare;
+  uint64_t calls = 0;          // launches through this cache
+  uint64_t last_eviction = 0;  // value of `calls` at the latest eviction
+  bool evicted_once = false;
+  // Entries are being evicted: launches get an event behind them.  Once the set of copies has
+  // settled (no eviction for a few hundred launches) the events stop again.
+  bool evicting() const { return evicted_once && calls - last_eviction < 4 * 64; }
 };
 int copy_cache(CopyCache** out) {
   static std::mutex mu;
@@ -381,6 +388,8 @@ int evict_one(CopyCache& c) {
   }
   if (victim.done) (void)hipEventDestroy(victim.done);
   if (victim.uploaded) (void)hipEventDestroy(victim.uploaded);
+  c.last_eviction = c.calls;
+  c.evicted_once = true;
   if (c.spare.size() < kSpareBufs) {
     c.spare.push_back(victim.buf);
   } else {
@@ -470,7 +479,8 @@ int mark_used(CopyCache& c, CachedCopy* entry, hipStream_t stream) {
   if (stream != entry->last_stream) entry->several_streams = true;
   entry->last_stream = stream;
   entry->done_is_latest = false;
-  if (c.lru.size() >= kCopyCacheCapacity) {
+  ++c.calls;
+  if (c.evicting()) {
     HVDHIP_CHECK(hipEventRecord(entry->done, stream));
     entry->done_is_latest = true;
   }
