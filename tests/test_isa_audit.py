@@ -1,0 +1,85 @@
+"""The generated gfx950 code of every kernel, checked without a GPU: the sources are compiled to
+assembly (hipcc cross-compiles here) and the text is searched for what must not be there.
+
+* no flat loads or stores (table-derived addresses must stay in the global address space),
+* no scratch memory (no register spills in a streaming kernel),
+* no packed fp32 arithmetic (the build switches its formation off),
+* every 16-byte load of streamed data carries the non-temporal hint -- the compiler drops it
+  silently from a vector load that is only byte-aligned, which is why byte elements are read
+  through raw buffer loads -- except in the Adasum first pass that keeps its vectors cached on
+  purpose."""
+import os
+import re
+import shutil
+import subprocess
+from concurrent.futures import ThreadPoolExecutor
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "horovod_amd", "csrc")
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-mllvm", "-amdgpu-kernarg-preload-count=16", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+         "-S", "--cuda-device-only"]
+
+
+def _assembly(tmp, name):
+    out = os.path.join(tmp, name + ".s")
+    r = subprocess.run(["hipcc"] + FLAGS + ["-o", out, os.path.join(CSRC, name + ".hip")],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=600)
+    assert r.returncode == 0, r.stdout.decode(errors="replace")[-2000:]
+    return open(out).read()
+
+
+@pytest.fixture(scope="module")
+def kernels(tmp_path_factory):
+    """{kernel symbol: [instruction lines]} over the three kernel sources."""
+    if shutil.which("hipcc") is None:
+        pytest.skip("hipcc is not installed")
+    tmp = str(tmp_path_factory.mktemp("isa"))
+    with ThreadPoolExecutor(3) as pool:
+        texts = list(pool.map(lambda n: _assembly(tmp, n), ["xfer", "reduce", "adasum"]))
+    found = {}
+    for text in texts:
+        name = None
+        for line in text.splitlines():
+            m = re.match(r"^(_ZN6hvdhip\S+):\s*; @", line)
+            if m:
+                name = m.group(1)
+                found[name] = []
+            elif name and line.startswith("\t") and not line.lstrip().startswith((";", ".")):
+                found[name].append(line.strip())
+                if line.strip().startswith("s_endpgm"):
+                    name = None
+    assert len(found) > 200, len(found)  # every instantiation of the three kernel families
+    return found
+
+
+def test_no_flat_scratch_or_packed_fp32(kernels):
+    for name, lines in kernels.items():
+        for ins in lines:
+            op = ins.split()[0]
+            assert not op.startswith(("flat_load", "flat_store")), (name, ins)
+            assert not op.startswith("scratch_"), (name, ins)
+            assert not re.match(r"v_pk_\w+_f32", op), (name, ins)
+
+
+def test_streaming_loads_keep_the_non_temporal_hint(kernels):
+    checked = 0
+    for name, lines in kernels.items():
+        if "finalize_k" in name:
+            continue  # reads the small table of partial sums, nothing streamed
+        keeps = "dot_partials_k" in name and name.split("dot_partials_kI")[1].split("EE")[0].endswith("Lb1")
+        # the fused scaled add also reads its layer's partial sums (24 bytes each, two per lane): not streamed
+        fused = re.search(r"scaled_add_kI\w+?Lb1ELb[01]EEE", name) is not None
+        plain = 0
+        for ins in lines:
+            op = ins.split()[0]
+            if op in ("global_load_dwordx4", "buffer_load_dwordx4"):
+                checked += 1
+                if keeps:
+                    assert " nt" not in ins, (name, ins)
+                elif " nt" not in ins:
+                    plain += 1
+        assert plain <= (4 if fused else 0), (name, plain)
+    assert checked > 1000, checked
