@@ -83,3 +83,26 @@ def test_streaming_loads_keep_the_non_temporal_hint(kernels):
                     plain += 1
         assert plain <= (4 if fused else 0), (name, plain)
     assert checked > 1000, checked
+
+
+def test_streaming_stores_carry_one_of_the_two_policies(kernels):
+    """Vector stores of streamed data are non-temporal global stores or write-through buffer
+    stores (sc0 sc1); a plain store would leave its lines in L2 for neither reader."""
+    checked = 0
+    for name, lines in kernels.items():
+        if "finalize_k" in name:
+            continue  # stores a layer's sums and coefficients, nothing streamed
+        streams_halves = "PackF32F16" in name  # the narrowing pack stores 8 bytes per lane
+        # sums and coefficients of a layer or chunk, written by one lane
+        small_results = 4 if ("scaled_add_k" in name or "dot_partials_k" in name) else 0
+        plain = 0
+        for ins in lines:
+            op = ins.split()[0]
+            if op == "global_store_dwordx4" or (streams_halves and op == "global_store_dwordx2"):
+                checked += 1
+                plain += " nt" not in ins
+            elif op in ("buffer_store_dwordx4", "buffer_store_dwordx2"):
+                checked += 1
+                assert " sc0 sc1" in ins and " nt" not in ins, (name, ins)
+        assert plain <= small_results, (name, plain)
+    assert checked > 1000, checked
