@@ -120,6 +120,17 @@ def test_more_entries_than_the_reference_batch_capacity(gpu, orc):
     _check_round_trip(gpu, orc, counts, F32, 0.125, 1.0, seed=5)
 
 
+@pytest.mark.parametrize("dtype", [F16, F32])
+def test_twenty_thousand_tiny_tensors(gpu, orc, dtype):
+    """A response of very many very small tensors (0 to 40 elements, so most are shorter than
+    the 16-byte pad unit and none fills a vector loop), packed misaligned to both sides."""
+    rng = np.random.default_rng(21)
+    counts = [int(c) for c in rng.integers(0, 41, 20000)]
+    es = SIZE_OF[dtype]
+    _check_round_trip(gpu, orc, counts, dtype, 0.125, 3.0, misalign=[0, es, 2 * es, 3 * es],
+                      out_misalign=[3 * es, 0, es], seed=22)
+
+
 def test_in_place_outputs_alias_tensors(gpu, orc):
     # allreduce_async_ passes output == tensor (torch/mpi_ops.py:265)
     rng = np.random.default_rng(6)
