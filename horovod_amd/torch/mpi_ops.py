@@ -364,10 +364,79 @@ def sparse_allreduce_async(tensor, name, op):
     return handle
 
 
+class _Broadcast:
+    """A broadcast in the simulated world: nothing travels, the value is already in place."""
+
+    def __init__(self, output):
+        self.output = output
+
+
+def broadcast_async_(tensor, root_rank, name=None):
+    """In-place broadcast from root_rank (horovod/torch/mpi_ops.py:645-690).  This process is rank 0
+    of the simulated world: with root 0 the tensor already holds the root's value; another
+    root's value comes from peer_source.  No kernel of the library is involved (in the
+    reference a broadcast has no fusion buffer either, ops/nccl_operations.cc:444-480)."""
+    eng = _state()
+    if not 0 <= root_rank < eng.size:
+        raise ValueError('Invalid root rank %d for a world of %d ranks.' % (root_rank, eng.size))
+    if root_rank != 0 and eng.peer_source is not None:
+        value = eng.peer_source(root_rank, _name(name, 'broadcast'), tensor)
+        if value.shape != tensor.shape or value.dtype != tensor.dtype:
+            raise HorovodInternalError('Mismatched broadcast tensor shapes or types for %r.' % name)
+        with torch.no_grad():
+            tensor.copy_(value)
+    handle = _next_handle[0] = _next_handle[0] + 1
+    _handle_map[handle] = _Broadcast(tensor)
+    return handle
+
+
+def broadcast_async(tensor, root_rank, name=None):
+    return broadcast_async_(tensor.clone(), root_rank, name)
+
+
+def broadcast_(tensor, root_rank, name=None):
+    return synchronize(broadcast_async_(tensor, root_rank, name))
+
+
+def broadcast(tensor, root_rank, name=None):
+    return synchronize(broadcast_async(tensor, root_rank, name))
+
+
+def broadcast_parameters(params, root_rank):
+    """horovod/torch/functions.py:28-59: a dict (state_dict), or a list of parameters or of
+    (name, parameter) pairs."""
+    if isinstance(params, dict):
+        params = sorted(params.items())
+    elif isinstance(params, list):
+        params = [p if isinstance(p, tuple) else (None, p) for p in params]
+    else:
+        raise ValueError('invalid params of type: %s' % type(params))
+    for handle in [broadcast_async_(p, root_rank, name) for name, p in params if isinstance(p, torch.Tensor)]:
+        synchronize(handle)
+
+
+def broadcast_optimizer_state(optimizer, root_rank):
+    """horovod/torch/functions.py:62-187.  The simulated ranks hold no optimizer, so only rank 0,
+    this process, can be the root, and then its state is already the state of the world."""
+    if root_rank != 0:
+        raise NotImplementedError('only rank 0 holds an optimizer in the simulated world')
+    _state()
+
+
+def broadcast_object(obj, root_rank=0, name=None):
+    """horovod/torch/functions.py:190-230."""
+    if root_rank != 0:
+        raise NotImplementedError('only rank 0 holds Python objects in the simulated world')
+    _state()
+    return obj
+
+
 def poll(handle):
     """True once the operation behind the handle has completed on the GPU; does not block."""
     if handle not in _handle_map:
         raise ValueError('Did not find a handle produced by an async operation.')  # mpi_ops.py poll()
+    if isinstance(_handle_map[handle], _Broadcast):
+        return True
     return _state().poll(_handle_map[handle])
 
 
@@ -376,6 +445,8 @@ def synchronize(handle):
     if handle not in _handle_map:
         return None
     req = _handle_map.pop(handle)
+    if isinstance(req, _Broadcast):
+        return req.output
     _state().wait(req)
     outs = [e.output for e in req.entries]
     return outs if req.grouped else outs[0]

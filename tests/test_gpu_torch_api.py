@@ -440,3 +440,31 @@ def test_adasum_against_the_reference_tests_numpy_tree(hvd, size, local_size):
             want = _reference_tree_reduction(sums) / local_size
             assert got.dtype == dtype
             assert np.allclose(got.double().cpu().numpy(), want, rtol=tol, atol=tol), (dtype, size, local_size)
+
+
+def test_broadcast_in_the_simulated_world(hvd):
+    """What a training script does before its first step (broadcast_parameters,
+    broadcast_optimizer_state from rank 0) is the identity here; another root's value comes from
+    peer_source."""
+    def peer(rank, name, tensor):
+        return torch.full_like(tensor, float(rank))
+
+    hvd.init(size=4, peer_source=peer)
+    model = torch.nn.Linear(3, 2).cuda()
+    before = {k: v.clone() for k, v in model.state_dict().items()}
+    hvd.broadcast_parameters(model.state_dict(), root_rank=0)
+    hvd.broadcast_parameters(list(model.named_parameters()), root_rank=0)
+    opt = torch.optim.SGD(model.parameters(), lr=0.1, momentum=0.9)
+    hvd.broadcast_optimizer_state(opt, root_rank=0)
+    assert hvd.broadcast_object({"epoch": 3}, root_rank=0) == {"epoch": 3}
+    for k, v in model.state_dict().items():
+        assert torch.equal(v, before[k])
+    t = torch.zeros(5, device="cuda")
+    out = hvd.broadcast(t, root_rank=2, name="b")
+    assert torch.equal(out, torch.full_like(t, 2.0)) and torch.equal(t, torch.zeros_like(t))
+    h = hvd.broadcast_async_(t, root_rank=3, name="c")
+    assert hvd.poll(h) and hvd.synchronize(h) is t and torch.equal(t, torch.full_like(t, 3.0))
+    with pytest.raises(ValueError, match="root rank"):
+        hvd.broadcast_(t, root_rank=4)
+    with pytest.raises(NotImplementedError):
+        hvd.broadcast_optimizer_state(opt, root_rank=1)
