@@ -4,6 +4,7 @@ assembly (hipcc cross-compiles here) and the text is searched for what must not 
 * no flat loads or stores (table-derived addresses must stay in the global address space),
 * no scratch memory (no register spills in a streaming kernel),
 * no packed fp32 arithmetic (the build switches its formation off),
+* no loop that makes a buffer resource uniform lane by lane (the windows' bases are uniform),
 * every 16-byte load of streamed data carries the non-temporal hint -- the compiler drops it
   silently from a vector load that is only byte-aligned, which is why byte elements are read
   through raw buffer loads -- except in the Adasum first pass that keeps its vectors cached on
@@ -59,6 +60,8 @@ def test_no_flat_scratch_or_packed_fp32(kernels):
     for name, lines in kernels.items():
         for ins in lines:
             op = ins.split()[0]
+            # a buffer resource that the compiler cannot prove uniform is made uniform in a loop
+            assert not op.startswith("v_readfirstlane"), (name, ins)
             assert not op.startswith(("flat_load", "flat_store")), (name, ins)
             assert not op.startswith("scratch_"), (name, ins)
             assert not re.match(r"v_pk_\w+_f32", op), (name, ins)
