@@ -2,7 +2,7 @@
 import ctypes
 import os
 from ctypes import (POINTER, c_char_p, c_double, c_float, c_int, c_int64, c_size_t,
-                    c_uint, c_void_p)
+                    c_uint, c_uint64, c_void_p)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
@@ -59,6 +59,8 @@ _PROTOTYPES = {
     "hvdhip_timer_destroy": (c_int, [c_void_p]),
     "hvdhip_batched_d2d_memcpy": (c_int, [_PV, _PV, POINTER(c_size_t), c_int, c_void_p]),
     "hvdhip_batched_scaled_d2d_memcpy": (c_int, [_PV, _PV, POINTER(c_size_t), c_int, c_double, c_int, c_void_p]),
+    "hvdhip_copy_cache_stats": (c_int, [POINTER(c_uint64)] * 4),
+    "hvdhip_copy_cache_set_limits": (c_int, [c_uint64, c_uint64]),
     "hvdhip_scale_buffer": (c_int, [c_void_p, c_void_p, c_int64, c_double, c_int, c_void_p]),
     "hvdhip_fusion_plan_create": (c_int, [_PV, _PV, POINTER(c_int64), c_int, c_int, c_int, _PV]),
     "hvdhip_fusion_plan_destroy": (c_int, [c_void_p]),

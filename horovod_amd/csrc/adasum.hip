@@ -23,7 +23,6 @@
 // loop.  Bandwidth-bound: 3 double fmas per 8 bytes read in pass 1.
 #include <cfloat>
 #include <cmath>
-#include <cstdlib>
 #include <list>
 #include <mutex>
 
@@ -177,11 +176,16 @@ __global__ __launch_bounds__(kWG) void finalize_k(const Layer* __restrict__ laye
   }
 }
 
-// ScaledAdd<T>, adasum.h:429-435: operands widened to double, one rounding.
+// ScaledAdd<T>, adasum.h:429-435: acoeff * a[i] + bcoeff * b[i] with the operands widened to
+// double: two rounded products, their rounded sum, then the conversion to T.  Contraction is
+// switched off for this expression (device code contracts by default, and the rounded-operation
+// intrinsics are plain operators to the compiler), so no product is fused into the sum.
 template <typename T>
 struct Axpby {
   static __device__ __forceinline__ T f(double ca, T a, double cb, T b) {
-    return (T)fma(ca, (double)a, cb * (double)b);
+#pragma clang fp contract(off)
+    const double pa = ca * (double)a, pb = cb * (double)b;
+    return (T)(pa + pb);
   }
 };
 // ScaledAddfp16, adasum.h:482-500: float coefficients, t = ca*a rounded to
@@ -339,14 +343,8 @@ namespace {
 // the 256 MB Infinity Cache by then, the first pass loads it without the non-temporal hint so
 // that it is kept: measured on the combine, +28 % at 2 x 16 MiB, +10 % at 2 x 32 MiB,
 // +6 % at 2 x 64 MiB and +2.5 % at 2 x 128 MiB; at 2 x 256 MiB it costs 0.8 % and beyond that nothing is left of it.
-// HVDHIP_ADASUM_KEEP_BYTES overrides the largest pair (both vectors, bytes) that is kept.
-uint64_t keep_cached_bytes() {
-  static const uint64_t limit = [] {
-    const char* e = std::getenv("HVDHIP_ADASUM_KEEP_BYTES");
-    return e ? (uint64_t)std::strtoull(e, nullptr, 0) : (uint64_t)320 << 20;
-  }();
-  return limit;
-}
+// The largest pair (both vectors, bytes) that is kept:
+constexpr uint64_t kKeepCachedBytes = (uint64_t)320 << 20;
 
 template <bool KEEP>
 void launch_dot_partials(hvdhip_adasum_plan* p, const void* a, const void* b, hipStream_t s) {
@@ -373,7 +371,7 @@ int plan_dot_norms(hvdhip_adasum_plan* p, const void* a, const void* b, hipStrea
   if (p->nlayers == 0) return 0;
   const DevTables& t = p->tables;
   if (t.nchunks > 0) {
-    if (2 * (uint64_t)p->total * (uint64_t)dtype_size(p->dtype) <= keep_cached_bytes())
+    if (2 * (uint64_t)p->total * (uint64_t)dtype_size(p->dtype) <= kKeepCachedBytes)
       launch_dot_partials<true>(p, a, b, s);
     else
       launch_dot_partials<false>(p, a, b, s);
@@ -419,15 +417,11 @@ int plan_scaled_add(hvdhip_adasum_plan* p, void* a, const void* b, const double*
   return scaled_add_by_dtype<false>(p, a, b, coeffs, ca, cb, s);
 }
 
-// The combine may leave the layer sums to the scaled add when every layer's partial triples
-// fit the two loads per lane that kernel spends on them and there is a workgroup to do it.
-// HVDHIP_ADASUM_FUSED_COEFFS=0 keeps the separate finalize launch, for comparison.
-bool fused_coeffs_enabled() {
-  static const bool on = [] {
-    const char* e = std::getenv("HVDHIP_ADASUM_FUSED_COEFFS");
-    return !(e && e[0] == '0');
-  }();
-  return on;
+// The combine leaves the layer sums to the scaled add when every layer's partial triples fit the
+// two loads per lane that kernel spends on them and there is a workgroup to do it (worth 0.6 % at
+// 64 layers of 2^25 elements, 3.5 % at 1,000 layers, 9 % at 2^22 elements).
+bool fused_coeffs(const hvdhip_adasum_plan* p) {
+  return p->tables.nchunks > 0 && p->max_layer_chunks <= 2 * (uint32_t)kWG;
 }
 
 int check_vectors(const hvdhip_adasum_plan* p, const void* a, const void* b) {
@@ -440,10 +434,19 @@ int check_vectors(const hvdhip_adasum_plan* p, const void* a, const void* b) {
   return 0;
 }
 
-// Single-layer plans for the Dispatch* entry points, keyed by (count, dtype).
+// Single-layer plans for the Dispatch* entry points, keyed by (count, dtype, device, stream): a
+// plan carries the partial sums of the launch that is using it, and callers on different streams
+// must not share those.  The cache's mutex is held for lookup and insertion only; an entry is
+// pinned by a use count while its caller launches on it and (for the blocking entry point)
+// waits for the result, and pinned entries are neither handed to a second caller nor evicted.
+struct OneLayerEntry {
+  hvdhip_adasum_plan* plan = nullptr;
+  hipStream_t stream = nullptr;
+  int users = 0;
+};
 struct OneLayerCache {
   std::mutex mu;
-  std::list<hvdhip_adasum_plan*> lru;
+  std::list<OneLayerEntry> lru;
 };
 OneLayerCache& one_layer_cache() {
   static OneLayerCache* c = new OneLayerCache();
@@ -451,29 +454,54 @@ OneLayerCache& one_layer_cache() {
 }
 constexpr size_t kOneLayerCapacity = 256;
 
-// The caller holds the cache mutex until its work on the plan is queued (and, for the
-// blocking entry point, finished): eviction destroys plans, and plans carry state.
-int one_layer_plan(int count, int dtype, hvdhip_adasum_plan** out) {
+// Pins a plan for (count, dtype) on the current device and `stream`; release with unpin().
+int pin_one_layer_plan(int count, int dtype, hipStream_t stream, OneLayerEntry** out) {
   OneLayerCache& c = one_layer_cache();
   int device = 0;
   HVDHIP_CHECK(hipGetDevice(&device));
-  for (auto it = c.lru.begin(); it != c.lru.end(); ++it) {
-    if ((*it)->total == count && (*it)->dtype == dtype && (*it)->device == device) {
-      c.lru.splice(c.lru.begin(), c.lru, it);
-      *out = c.lru.front();
-      return 0;
+  {
+    std::lock_guard<std::mutex> g(c.mu);
+    for (auto it = c.lru.begin(); it != c.lru.end(); ++it) {
+      if (it->users == 0 && it->stream == stream && it->plan->total == count && it->plan->dtype == dtype &&
+          it->plan->device == device) {
+        c.lru.splice(c.lru.begin(), c.lru, it);
+        ++c.lru.front().users;
+        *out = &c.lru.front();
+        return 0;
+      }
     }
   }
+  // building a plan allocates and synchronises: outside the mutex
   hvdhip_adasum_plan* p = nullptr;
   int rc = hvdhip_adasum_plan_create(&count, 1, dtype, &p);
   if (rc) return rc;
-  if (c.lru.size() >= kOneLayerCapacity) {
-    hvdhip_adasum_plan_destroy(c.lru.back());
-    c.lru.pop_back();
+  hvdhip_adasum_plan* victim = nullptr;
+  {
+    std::lock_guard<std::mutex> g(c.mu);
+    if (c.lru.size() >= kOneLayerCapacity) {
+      for (auto it = c.lru.end(); it != c.lru.begin();) {
+        --it;
+        if (it->users == 0) {
+          victim = it->plan;
+          c.lru.erase(it);
+          break;
+        }
+      }
+    }
+    OneLayerEntry e;
+    e.plan = p;
+    e.stream = stream;
+    e.users = 1;
+    c.lru.push_front(e);
+    *out = &c.lru.front();  // list nodes do not move
   }
-  c.lru.push_front(p);
-  *out = p;
+  if (victim) hvdhip_adasum_plan_destroy(victim);  // waits for the device: outside the mutex
   return 0;
+}
+
+void unpin(OneLayerEntry* e) {
+  std::lock_guard<std::mutex> g(one_layer_cache().mu);
+  --e->users;
 }
 
 }  // namespace
@@ -575,8 +603,7 @@ int hvdhip_adasum_combine(hvdhip_adasum_plan* plan, void* a, const void* b, void
   int rc = check_vectors(plan, a, b);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool fused = plan->tables.nchunks > 0 && plan->max_layer_chunks <= 2 * (uint32_t)kWG &&
-                     fused_coeffs_enabled();
+  const bool fused = fused_coeffs(plan);
   rc = plan_dot_norms(plan, a, b, s, !fused);
   if (rc) return rc;
   rc = fused ? scaled_add_by_dtype<true>(plan, a, b, nullptr, 0., 0., s)
@@ -616,16 +643,14 @@ int hvdhip_adasum_dot_and_norm_sqrds(const void* a, const void* b, int dtype, in
                                      void* stream) {
   if (!dot || !anormsq || !bnormsq) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "result pointer is NULL");
   if (count < 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "count is negative");
-  hvdhip_adasum_plan* p = nullptr;
-  std::lock_guard<std::mutex> g(one_layer_cache().mu);
-  int rc = one_layer_plan(count, dtype, &p);
+  OneLayerEntry* e = nullptr;
+  int rc = pin_one_layer_plan(count, dtype, static_cast<hipStream_t>(stream), &e);
   if (rc) return rc;
-  rc = check_vectors(p, a, b);
-  if (rc) return rc;
-  rc = plan_dot_norms(p, a, b, static_cast<hipStream_t>(stream));
-  if (rc) return rc;
-  double out[3];
-  rc = hvdhip_adasum_read(p, out, nullptr, stream);
+  double out[3] = {0., 0., 0.};
+  rc = check_vectors(e->plan, a, b);
+  if (rc == 0) rc = plan_dot_norms(e->plan, a, b, static_cast<hipStream_t>(stream));
+  if (rc == 0) rc = hvdhip_adasum_read(e->plan, out, nullptr, stream);  // blocks; the mutex is not held
+  unpin(e);
   if (rc) return rc;
   *dot = out[0];
   *anormsq = out[1];
@@ -636,13 +661,12 @@ int hvdhip_adasum_dot_and_norm_sqrds(const void* a, const void* b, int dtype, in
 int hvdhip_adasum_dispatch_scaled_add(int dtype, int count, double acoeff, void* a,
                                       double bcoeff, const void* b, void* stream) {
   if (count < 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "count is negative");
-  hvdhip_adasum_plan* p = nullptr;
-  std::lock_guard<std::mutex> g(one_layer_cache().mu);
-  int rc = one_layer_plan(count, dtype, &p);
+  OneLayerEntry* e = nullptr;
+  int rc = pin_one_layer_plan(count, dtype, static_cast<hipStream_t>(stream), &e);
   if (rc) return rc;
-  rc = check_vectors(p, a, b);
-  if (rc) return rc;
-  rc = plan_scaled_add(p, a, b, nullptr, acoeff, bcoeff, static_cast<hipStream_t>(stream));
+  rc = check_vectors(e->plan, a, b);
+  if (rc == 0) rc = plan_scaled_add(e->plan, a, b, nullptr, acoeff, bcoeff, static_cast<hipStream_t>(stream));
+  unpin(e);
   return rc ? rc : ok();
 }
 

@@ -119,11 +119,6 @@ uint64_t count_chunks(const std::vector<Seg>& segs, uint32_t chunk_units) {
 }
 
 uint32_t xcd_run(uint64_t nchunks, uint32_t chunk_bytes, bool long_runs) {
-  static const long forced = [] {
-    const char* e = std::getenv("HVDHIP_XCD_RUN");
-    return e ? std::strtol(e, nullptr, 10) : -1L;
-  }();
-  if (forced >= 0) return (uint32_t)forced;
   if (chunk_bytes == 0) return 0;
   const uint32_t bytes =
       !long_runs && nchunks * (uint64_t)chunk_bytes <= kXcdLongRunFrom ? kXcdRunBytes : kXcdLongRunBytes;
@@ -260,6 +255,10 @@ int hvdhip_stream_destroy(void* stream) {
     }
     p.filled.erase(key);
   }
+  // Work still queued completes first, so that nothing the library remembers about the stream
+  // (tables a launch on it reads) outlives it.
+  HVDHIP_CHECK(hipStreamSynchronize(s));
+  copy_cache_forget_stream(s);
   HVDHIP_CHECK(hipStreamDestroy(s));
   return ok();
 }

@@ -87,8 +87,7 @@ uint32_t chunk_bytes(Family f);
 // a run in bytes.  Measured against natural order: 256 KiB per run is best for launches of 16-128
 // MiB (+2-5 % on every kernel family; 128 KiB - 1 MiB are close, a single chunk and >= 4 MiB gain
 // nothing) but costs 2-6 % at 512 MiB and more, where 1 MiB gains 1-3 % and 4 MiB loses 4-6 %; so
-// launches that cover more than kXcdLongRunFrom bytes use the longer run.  HVDHIP_XCD_RUN overrides
-// the run length (in chunks) for every launch, 0 switches the reordering off.
+// launches that cover more than kXcdLongRunFrom bytes use the longer run.
 constexpr uint32_t kXcds = 8;
 constexpr uint32_t kXcdRunBytes = 256u << 10;
 constexpr uint32_t kXcdLongRunBytes = 1u << 20;
@@ -216,6 +215,9 @@ class DeviceGuard {
   int prev_ = 0;
   bool switched_ = false;
 };
+
+// Tells the copy-table caches that `stream` has been synchronised and is about to be destroyed.
+void copy_cache_forget_stream(hipStream_t stream);
 
 // Uploads a ready-made chunk table.
 int upload_chunks(const std::vector<Chunk>& chunks, DevTables* out);

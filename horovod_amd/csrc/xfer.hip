@@ -28,9 +28,12 @@
 // scaled in double and truncated toward zero.
 #include <algorithm>
 #include <cstring>
+#include <deque>
+#include <iterator>
 #include <list>
 #include <map>
 #include <mutex>
+#include <unordered_map>
 
 #include "internal.h"
 #include "vecmem.h"
@@ -287,18 +290,21 @@ int launch_contig(const void* in, void* out, int64_t n, typename Op::P p, hipStr
 // ---- cache of tables for the array-taking entry points ----------------
 //
 // The reference passes its copy descriptors by value with every launch, so a
-// caller of these entry points expects no set-up cost.  A hit costs a key
-// comparison.  A miss allocates nothing and never waits for the device in the
-// steady state: the table is written straight into a pinned staging buffer
-// that belongs to the cache entry, copied to the entry's device buffer with an
-// asynchronous copy on the caller's stream, and the kernel follows on the
-// same stream.  Evicted entries hand their buffers to the next miss; before
-// that, the entry's last-use event is waited for (normally long complete).
-// That event costs a command on the stream after every launch (about 3 us
-// between two 17 us copies), so it is only recorded while the cache is full
-// and entries are being evicted (or were, within the last 256 launches); a
-// victim whose last use went unrecorded makes the eviction wait for the whole
-// device once.
+// caller of these entry points expects no set-up cost.  The cache keeps one
+// device-resident table per distinct (out, in, sizes) set, found through a hash
+// of the arrays; a hit costs the hash and one comparison.  It grows with the
+// number of sets a job cycles through (a GPT-2 XL step has 49 fusion cycles
+// times two directions) and is bounded by the device memory its tables take,
+// not by a count of entries.
+//
+// A miss never waits for the device: the table is written into a pinned staging
+// buffer that belongs to the entry, copied to the entry's device buffer with an
+// asynchronous copy on the caller's stream, and the kernel follows on the same
+// stream.  Launches leave nothing behind on the stream; an entry only remembers
+// which streams have read its table.  When an entry is evicted, an event is
+// recorded at the current tail of each of those streams and the entry's buffers
+// are retired with those events; a later miss reuses retired buffers whose
+// events have completed and allocates new ones otherwise.
 
 struct TableBuf {
   void* dev = nullptr;
@@ -307,15 +313,20 @@ struct TableBuf {
 };
 
 struct CachedCopy {
+  uint64_t hash = 0;
   std::vector<uint64_t> key;  // unit size, n, then out/in/size triples
   DevTables tables;           // tables.alloc is not owned: it aliases buf.dev
   TableBuf buf;
   hipEvent_t uploaded = nullptr;    // recorded once, behind the table's upload on the stream that built it
   bool upload_complete = false;     // `uploaded` has been seen complete: other streams need not wait for it
-  hipEvent_t done = nullptr;        // recorded after a launch that reads the table, while the cache is full
-  bool done_is_latest = false;      // the latest launch was followed by a record of `done`
-  hipStream_t last_stream = nullptr;
-  bool several_streams = false;     // used on more than one stream since it was built
+  hipStream_t build_stream = nullptr;
+  std::vector<hipStream_t> streams;  // every stream that holds, or held, a launch reading the table
+};
+
+// Buffers of an evicted entry; free for reuse once every event has completed.
+struct Retired {
+  TableBuf buf;
+  std::vector<hipEvent_t> events;
 };
 
 // One cache per device: its entries, their buffers and the spare buffers all live on that
@@ -323,27 +334,35 @@ struct CachedCopy {
 struct CopyCache {
   std::mutex mu;
   std::list<CachedCopy> lru;  // front = most recent
+  std::unordered_multimap<uint64_t, std::list<CachedCopy>::iterator> index;  // by CachedCopy::hash
   std::vector<TableBuf> spare;
-  uint64_t calls = 0;          // launches through this cache
-  uint64_t last_eviction = 0;  // value of `calls` at the latest eviction
-  bool evicted_once = false;
-  // Entries are being evicted: launches get an event behind them.  Once the set of copies has
-  // settled (no eviction for a few hundred launches) the events stop again.
-  bool evicting() const { return evicted_once && calls - last_eviction < 4 * 64; }
+  std::deque<Retired> retired;       // oldest first
+  std::vector<hipEvent_t> idle_events;
+  size_t bytes = 0;                  // device bytes of the live entries' tables
+  size_t max_entries = 4096;
+  size_t max_bytes = (size_t)256 << 20;
+  uint64_t hits = 0, misses = 0, evictions = 0;
 };
+struct CacheRegistry {
+  std::mutex mu;
+  std::map<int, CopyCache*> by_device;
+};
+CacheRegistry& registry() {
+  static CacheRegistry* r = new CacheRegistry();  // never destroyed: outlives static teardown
+  return *r;
+}
 int copy_cache(CopyCache** out) {
-  static std::mutex mu;
-  static std::map<int, CopyCache*>* caches = new std::map<int, CopyCache*>();  // never destroyed
   int device = 0;
   HVDHIP_CHECK(hipGetDevice(&device));
-  std::lock_guard<std::mutex> g(mu);
-  CopyCache*& c = (*caches)[device];
+  CacheRegistry& r = registry();
+  std::lock_guard<std::mutex> g(r.mu);
+  CopyCache*& c = r.by_device[device];
   if (!c) c = new CopyCache();
   *out = c;
   return 0;
 }
-constexpr size_t kCopyCacheCapacity = 64;
-constexpr size_t kSpareBufs = 8;
+constexpr size_t kSpareBufs = 16;
+constexpr size_t kMaxRetired = 64;
 
 void release_buf(TableBuf* b) {
   if (b->dev) (void)hipFree(b->dev);
@@ -351,8 +370,51 @@ void release_buf(TableBuf* b) {
   *b = TableBuf();
 }
 
+// Internal ordering only (table uploads and table reads): no timing, no system-scope fence.
+int order_event(CopyCache& c, hipEvent_t* out) {
+  if (!c.idle_events.empty()) {
+    *out = c.idle_events.back();
+    c.idle_events.pop_back();
+    return 0;
+  }
+  HVDHIP_CHECK(hipEventCreateWithFlags(out, hipEventDisableTiming | hipEventDisableSystemFence));
+  return 0;
+}
+
+void keep_buf(CopyCache& c, TableBuf* b) {
+  if (c.spare.size() < kSpareBufs) {
+    c.spare.push_back(*b);
+    *b = TableBuf();
+  } else {
+    release_buf(b);
+  }
+}
+
+// Moves retired buffers whose events have completed to the spares.  wait_oldest: block for the
+// oldest one's events first (only when too many are retired, which means the device is far behind).
+void reap_retired(CopyCache& c, bool wait_oldest) {
+  while (!c.retired.empty()) {
+    Retired& r = c.retired.front();
+    bool complete = true;
+    for (hipEvent_t e : r.events) {
+      hipError_t q = wait_oldest ? hipEventSynchronize(e) : hipEventQuery(e);
+      if (q != hipSuccess) {
+        (void)hipGetLastError();  // hipErrorNotReady is not an error here
+        complete = false;
+        break;
+      }
+    }
+    if (!complete) return;
+    for (hipEvent_t e : r.events) c.idle_events.push_back(e);
+    keep_buf(c, &r.buf);
+    c.retired.pop_front();
+    wait_oldest = false;
+  }
+}
+
 // A device + pinned buffer pair of at least `bytes`: the smallest spare that fits, else new.
 int acquire_buf(CopyCache& c, size_t bytes, TableBuf* out) {
+  reap_retired(c, c.retired.size() > kMaxRetired);
   size_t best = c.spare.size();
   for (size_t i = 0; i < c.spare.size(); ++i)
     if (c.spare[i].cap >= bytes && (best == c.spare.size() || c.spare[i].cap < c.spare[best].cap)) best = i;
@@ -377,26 +439,67 @@ int acquire_buf(CopyCache& c, size_t bytes, TableBuf* out) {
   return 0;
 }
 
-// Takes the least recently used entry out of the cache once nothing on the device can
-// still read its table, and keeps its buffers for reuse.
+// Takes the least recently used entry out of the cache.  Nothing is waited for: an event goes
+// behind whatever each stream that used the table holds now, and the buffers are retired with
+// those events.  A stream that no longer exists cannot take an event; its work is then waited
+// for with the rest of the device (a stream destroyed through hvdhip_stream_destroy has been
+// taken off every entry first, so this is left to foreign streams that were destroyed).
 int evict_one(CopyCache& c) {
-  CachedCopy& victim = c.lru.back();
-  if (victim.several_streams || !victim.done_is_latest) {
-    HVDHIP_CHECK(hipDeviceSynchronize());
-  } else {
-    HVDHIP_CHECK(hipEventSynchronize(victim.done));
+  auto victim = std::prev(c.lru.end());
+  Retired r;
+  r.buf = victim->buf;
+  bool lost_stream = false;
+  for (hipStream_t s : victim->streams) {
+    hipEvent_t e = nullptr;
+    int rc = order_event(c, &e);
+    if (rc) return rc;
+    if (hipEventRecord(e, s) == hipSuccess) {
+      r.events.push_back(e);
+    } else {
+      (void)hipGetLastError();
+      c.idle_events.push_back(e);
+      lost_stream = true;
+    }
   }
-  if (victim.done) (void)hipEventDestroy(victim.done);
-  if (victim.uploaded) (void)hipEventDestroy(victim.uploaded);
-  c.last_eviction = c.calls;
-  c.evicted_once = true;
-  if (c.spare.size() < kSpareBufs) {
-    c.spare.push_back(victim.buf);
-  } else {
-    release_buf(&victim.buf);
+  if (lost_stream) HVDHIP_CHECK(hipDeviceSynchronize());
+  if (victim->uploaded) r.events.push_back(victim->uploaded);  // the pinned half is read by the upload
+  c.retired.push_back(std::move(r));
+  c.bytes -= victim->buf.cap;
+  auto range = c.index.equal_range(victim->hash);
+  for (auto it = range.first; it != range.second; ++it) {
+    if (it->second == victim) {
+      c.index.erase(it);
+      break;
+    }
   }
-  c.lru.pop_back();
+  c.lru.erase(victim);
+  ++c.evictions;
   return 0;
+}
+
+uint64_t hash_arrays(void* const* out, const void* const* in, const size_t* sizes, int n, uint32_t unit) {
+  uint64_t h = 0x9e3779b97f4a7c15ull ^ ((uint64_t)unit << 32) ^ (uint64_t)n;
+  auto mix = [&h](uint64_t x) {
+    h ^= x;
+    h *= 0xff51afd7ed558ccdull;
+    h ^= h >> 32;
+  };
+  for (int i = 0; i < n; ++i) {
+    mix((uint64_t)(uintptr_t)out[i]);
+    mix((uint64_t)(uintptr_t)in[i]);
+    mix((uint64_t)sizes[i]);
+  }
+  return h;
+}
+
+bool same_arrays(const std::vector<uint64_t>& key, void* const* out, const void* const* in,
+                 const size_t* sizes, int n, uint32_t unit) {
+  if (key.size() != 2 + 3 * (size_t)n || key[0] != unit || key[1] != (uint64_t)n) return false;
+  const uint64_t* k = key.data() + 2;
+  for (int i = 0; i < n; ++i, k += 3)
+    if (k[0] != (uint64_t)(uintptr_t)out[i] || k[1] != (uint64_t)(uintptr_t)in[i] || k[2] != (uint64_t)sizes[i])
+      return false;
+  return true;
 }
 
 // Finds or builds the table for (out, in, sizes) with elements of unit bytes; a newly
@@ -404,32 +507,25 @@ int evict_one(CopyCache& c) {
 // launches on `stream`, then calls mark_used() before releasing the mutex.
 int cached_tables(CopyCache& c, void* const* out, const void* const* in, const size_t* sizes, int n,
                   uint32_t unit, hipStream_t stream, CachedCopy** result) {
-  std::vector<uint64_t> key;
-  key.reserve(2 + 3 * (size_t)n);
-  key.push_back((uint64_t)unit);
-  key.push_back((uint64_t)n);
-  for (int i = 0; i < n; ++i) {
-    key.push_back((uint64_t)(uintptr_t)out[i]);
-    key.push_back((uint64_t)(uintptr_t)in[i]);
-    key.push_back((uint64_t)sizes[i]);
-  }
-  for (auto it = c.lru.begin(); it != c.lru.end(); ++it) {
-    if (it->key == key) {
-      c.lru.splice(c.lru.begin(), c.lru, it);
-      CachedCopy* hit = &c.lru.front();
-      // The table was uploaded asynchronously on the stream that built it; another stream
-      // must not read it earlier.
-      if (!hit->upload_complete) {
-        if (hipEventQuery(hit->uploaded) == hipSuccess) {
-          hit->upload_complete = true;
-        } else {
-          (void)hipGetLastError();  // hipErrorNotReady is not an error here
-          if (stream != hit->last_stream) HVDHIP_CHECK(hipStreamWaitEvent(stream, hit->uploaded, 0));
-        }
+  const uint64_t hash = hash_arrays(out, in, sizes, n, unit);
+  auto range = c.index.equal_range(hash);
+  for (auto it = range.first; it != range.second; ++it) {
+    if (!same_arrays(it->second->key, out, in, sizes, n, unit)) continue;
+    c.lru.splice(c.lru.begin(), c.lru, it->second);  // iterators into a list survive a splice
+    CachedCopy* hit = &c.lru.front();
+    // The table was uploaded asynchronously on the stream that built it; another stream
+    // must not read it earlier.
+    if (!hit->upload_complete) {
+      if (hipEventQuery(hit->uploaded) == hipSuccess) {
+        hit->upload_complete = true;
+      } else {
+        (void)hipGetLastError();  // hipErrorNotReady is not an error here
+        if (stream != hit->build_stream) HVDHIP_CHECK(hipStreamWaitEvent(stream, hit->uploaded, 0));
       }
-      *result = hit;
-      return 0;
     }
+    ++c.hits;
+    *result = hit;
+    return 0;
   }
   std::vector<Seg> segs((size_t)n);
   for (int i = 0; i < n; ++i)
@@ -437,54 +533,55 @@ int cached_tables(CopyCache& c, void* const* out, const void* const* in, const s
   const uint32_t chunk_units = chunk_bytes(Family::kXfer) / unit;
   const uint64_t nchunks = count_chunks(segs, chunk_units);
   if (nchunks == ~0ull) return fail(HVDHIP_ERR_TOO_LARGE, "the copies need more than 2^23 workgroups");
-  if (c.lru.size() >= kCopyCacheCapacity) {
+  const size_t bytes = (size_t)nchunks * sizeof(Chunk);
+  while (!c.lru.empty() && (c.lru.size() >= c.max_entries || c.bytes + bytes > c.max_bytes)) {
     int rc = evict_one(c);
     if (rc) return rc;
   }
   CachedCopy entry;
-  const size_t bytes = (size_t)nchunks * sizeof(Chunk);
   int rc = acquire_buf(c, bytes ? bytes : 32, &entry.buf);
   if (rc) return rc;
-  // internal ordering only (table uploads and table reads): no timing, no system-scope fence
-  constexpr unsigned kOrderOnly = hipEventDisableTiming | hipEventDisableSystemFence;
-  hipError_t e = hipEventCreateWithFlags(&entry.done, kOrderOnly);
-  if (e == hipSuccess) e = hipEventCreateWithFlags(&entry.uploaded, kOrderOnly);
-  if (e == hipSuccess && nchunks) {
+  rc = order_event(c, &entry.uploaded);
+  hipError_t e = hipSuccess;
+  if (rc == 0 && nchunks) {
     fill_chunks(segs, chunk_units, unit, unit, static_cast<Chunk*>(entry.buf.pinned), nchunks);
     e = hipMemcpyAsync(entry.buf.dev, entry.buf.pinned, bytes, hipMemcpyHostToDevice, stream);
   }
-  if (e == hipSuccess) e = hipEventRecord(entry.uploaded, stream);
-  if (e != hipSuccess) {
+  if (rc == 0 && e == hipSuccess) e = hipEventRecord(entry.uploaded, stream);
+  if (rc || e != hipSuccess) {
     (void)hipGetLastError();
-    if (entry.done) (void)hipEventDestroy(entry.done);
-    if (entry.uploaded) (void)hipEventDestroy(entry.uploaded);
+    if (entry.uploaded) c.idle_events.push_back(entry.uploaded);
     // the copy may have been queued: do not hand the buffers on before the stream is idle
     (void)hipStreamSynchronize(stream);
-    c.spare.push_back(entry.buf);
-    return fail((int)e, "staging a copy table failed: %s", hipGetErrorString(e));
+    keep_buf(c, &entry.buf);
+    return rc ? rc : fail((int)e, "staging a copy table failed: %s", hipGetErrorString(e));
   }
-  entry.key.swap(key);
+  entry.hash = hash;
+  entry.key.reserve(2 + 3 * (size_t)n);
+  entry.key.push_back((uint64_t)unit);
+  entry.key.push_back((uint64_t)n);
+  for (int i = 0; i < n; ++i) {
+    entry.key.push_back((uint64_t)(uintptr_t)out[i]);
+    entry.key.push_back((uint64_t)(uintptr_t)in[i]);
+    entry.key.push_back((uint64_t)sizes[i]);
+  }
   entry.tables.alloc = nullptr;
   entry.tables.chunks = static_cast<Chunk*>(entry.buf.dev);
   entry.tables.nchunks = (uint32_t)nchunks;
-  entry.last_stream = stream;
+  entry.build_stream = stream;
+  c.bytes += entry.buf.cap;
   c.lru.push_front(std::move(entry));
+  c.index.emplace(hash, c.lru.begin());
+  ++c.misses;
   *result = &c.lru.front();
   return 0;
 }
 
-// Notes that `stream` now holds work reading the entry's table, with an event behind it while
-// the cache is full (the next miss will evict).
-int mark_used(CopyCache& c, CachedCopy* entry, hipStream_t stream) {
-  if (stream != entry->last_stream) entry->several_streams = true;
-  entry->last_stream = stream;
-  entry->done_is_latest = false;
-  ++c.calls;
-  if (c.evicting()) {
-    HVDHIP_CHECK(hipEventRecord(entry->done, stream));
-    entry->done_is_latest = true;
-  }
-  return 0;
+// Notes that `stream` now holds work reading the entry's table.
+void mark_used(CachedCopy* entry, hipStream_t stream) {
+  for (hipStream_t s : entry->streams)
+    if (s == stream) return;
+  entry->streams.push_back(stream);
 }
 
 int check_arrays(void* const* out, const void* const* in, const size_t* sizes, int n) {
@@ -497,6 +594,27 @@ int check_arrays(void* const* out, const void* const* in, const size_t* sizes, i
 }
 
 }  // namespace
+
+// The stream is idle and about to be destroyed: no table is read on it any more.
+void copy_cache_forget_stream(hipStream_t stream) {
+  std::vector<CopyCache*> caches;
+  {
+    CacheRegistry& r = registry();
+    std::lock_guard<std::mutex> g(r.mu);
+    for (auto& kv : r.by_device) caches.push_back(kv.second);
+  }
+  for (CopyCache* c : caches) {
+    std::lock_guard<std::mutex> g(c->mu);
+    for (CachedCopy& e : c->lru) {
+      e.streams.erase(std::remove(e.streams.begin(), e.streams.end(), stream), e.streams.end());
+      if (e.build_stream == stream) {
+        e.build_stream = nullptr;
+        e.upload_complete = true;  // the stream was synchronised before this call
+      }
+    }
+  }
+}
+
 }  // namespace hvdhip
 
 using namespace hvdhip;
@@ -528,9 +646,8 @@ int hvdhip_batched_d2d_memcpy(void* const* out, const void* const* in, const siz
   std::lock_guard<std::mutex> g(cache->mu);
   rc = cached_tables(*cache, out, in, sizes, num_copies, 1, s, &entry);
   if (rc) return rc;
+  mark_used(entry, s);
   rc = launch_xfer<Copy<uint8_t>, kDirect>(entry->tables, 0, {}, s);
-  int rc2 = mark_used(*cache, entry, s);
-  if (rc == 0) rc = rc2;
   return rc ? rc : ok();
 }
 
@@ -557,10 +674,36 @@ int hvdhip_batched_scaled_d2d_memcpy(void* const* out, const void* const* in,
   std::lock_guard<std::mutex> g(cache->mu);
   rc = cached_tables(*cache, out, in, sizes, num_copies, es, s, &entry);
   if (rc) return rc;
+  mark_used(entry, s);
   rc = launch_same_dtype<kDirect>(entry->tables, 0, scale_factor, dtype, s);
-  int rc2 = mark_used(*cache, entry, s);
-  if (rc == 0) rc = rc2;
   return rc ? rc : ok();
+}
+
+int hvdhip_copy_cache_stats(uint64_t* hits, uint64_t* misses, uint64_t* evictions, uint64_t* entries) {
+  CopyCache* cache = nullptr;
+  int rc = copy_cache(&cache);
+  if (rc) return rc;
+  std::lock_guard<std::mutex> g(cache->mu);
+  if (hits) *hits = cache->hits;
+  if (misses) *misses = cache->misses;
+  if (evictions) *evictions = cache->evictions;
+  if (entries) *entries = (uint64_t)cache->lru.size();
+  return ok();
+}
+
+int hvdhip_copy_cache_set_limits(uint64_t max_entries, uint64_t max_bytes) {
+  if (max_entries == 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "max_entries is zero");
+  CopyCache* cache = nullptr;
+  int rc = copy_cache(&cache);
+  if (rc) return rc;
+  std::lock_guard<std::mutex> g(cache->mu);
+  cache->max_entries = (size_t)max_entries;
+  cache->max_bytes = (size_t)max_bytes;
+  while (!cache->lru.empty() && (cache->lru.size() > cache->max_entries || cache->bytes > cache->max_bytes)) {
+    rc = evict_one(*cache);
+    if (rc) return rc;
+  }
+  return ok();
 }
 
 int hvdhip_scale_buffer(const void* fused_input_data, void* buffer_data, int64_t num_elements,

@@ -20,7 +20,7 @@ import torch
 
 from . import host as H
 from ._lib import check, dtype_size, lib
-from .workloads import FUSION_THRESHOLD, fuse
+from .workloads import FUSION_THRESHOLD, fuse, reduce_scatter_share
 
 
 class Cycle:
@@ -77,12 +77,17 @@ class AllreducePipeline:
         num_streams = len(self.streams)
         self.completion_events = (num_streams > 1) if completion_events is None else bool(completion_events)
         self.pending = []  # (stream, event) recorded after each cycle
-        self.buffers = [torch.empty(max(max_len, 16), dtype=torch.uint8, device="cuda") for _ in range(num_streams)]
+        # room for the dummy elements a reduce-scatter over up to 64 ranks may append (64 * 64 elements)
+        self.buffers = [torch.zeros(max(max_len, 16) + 4096 * bs, dtype=torch.uint8, device="cuda")
+                        for _ in range(num_streams)]
         torch.cuda.synchronize()
 
     def reduce_elems(self, cyc, fraction):
-        n = int(cyc.buffer_elems * fraction)
-        return max(n - n % 8, 0) if fraction < 1.0 else cyc.buffer_elems
+        """Elements of the chunk that is reduced: the whole buffer, or with fraction = 1 / world the
+        share of rank 0 in the reference's reduce-scatter (ops/nccl_operations.cc:289-316)."""
+        if fraction >= 1.0:
+            return cyc.buffer_elems
+        return reduce_scatter_share(cyc.buffer_elems, int(round(1.0 / fraction)), fused=cyc.plan is not None)
 
     def run(self, prescale, postscale, peer_ptr=None, num_peers=0, fraction=1.0, kway=True, flags=0):
         """Queues every cycle; returns without synchronising."""

@@ -243,18 +243,11 @@ class Engine:
             plan = self._plan([e.tensor.data_ptr() for _, e in group], [e.output.data_ptr() for _, e in group],
                               counts, tdt, wire)
             nbytes = plan.buffer_len
-            result = self._buffer(slot, 0, nbytes)
-            plan.pack(result, first.prescale, s, flags)
-            offsets = plan.offsets() + [nbytes]
-            layer_counts = [(offsets[i + 1] - offsets[i]) // es for i in range(len(group))]  # pad bytes are zero
         else:
-            e = group[0][1]
-            nbytes = e.count * es
-            result = e.output.data_ptr()
-            self._scale_or_copy(e.tensor.data_ptr(), result, e.count, first.prescale, tdt, s)
-            layer_counts = [e.count]
-        nelem = nbytes // es
+            nbytes = group[0][1].count * es
 
+        # The other ranks' buffers first: with peer_source=None they are made from this rank's own
+        # tensors, which an in-place request (output is tensor) overwrites below.
         peer_bufs = []
         for rank, tensors in enumerate(peers, start=1):
             pb = self._buffer(slot, rank, nbytes)
@@ -264,6 +257,18 @@ class Engine:
             else:
                 self._scale_or_copy(tensors[0].data_ptr(), pb, counts[0], first.prescale, tdt, s)
             peer_bufs.append(pb)
+
+        if fused:
+            result = self._buffer(slot, 0, nbytes)
+            plan.pack(result, first.prescale, s, flags)
+            offsets = plan.offsets() + [nbytes]
+            layer_counts = [(offsets[i + 1] - offsets[i]) // es for i in range(len(group))]  # pad bytes are zero
+        else:
+            e = group[0][1]
+            result = e.output.data_ptr()
+            self._scale_or_copy(e.tensor.data_ptr(), result, e.count, first.prescale, tdt, s)
+            layer_counts = [e.count]
+        nelem = nbytes // es
 
         if nelem and peer_bufs:
             if first.op == ADASUM:

@@ -84,6 +84,22 @@ def numel(shape):
     return n
 
 
+FUSION_BUFFER_ATOMIC_UNIT = 64  # common/common.h:146
+
+
+def reduce_scatter_share(num_elements, world, fused=True):
+    """Elements of one GPU's share of the reduce-scatter over a buffer of num_elements, as
+    NCCLHierarchicalAllreduce::Execute cuts it (ops/nccl_operations.cc:285-316).  A fused response
+    first grows to a multiple of world * 64 elements (the extra ones are dummy elements behind the
+    payload, inside the fusion buffer, whose size the planner keeps divisible); every rank then owns
+    num_elements / world consecutive elements starting at rank * share.  A single tensor is not
+    grown: its remainder num_elements % world goes through a separate reduce at the last rank."""
+    if fused:
+        div = world * FUSION_BUFFER_ATOMIC_UNIT
+        num_elements = (num_elements + div - 1) // div * div
+    return num_elements // world
+
+
 def fuse(nbytes, threshold=FUSION_THRESHOLD, pad16=True):
     """Greedy fusion of a list of tensor byte sizes (one dtype, one set of scale
     factors) into groups of tensor indices, in the reference's queue discipline."""

@@ -168,9 +168,22 @@ int hvdhip_timer_destroy(void* timer);
  * BatchedD2DParams); there is no 160-entry limit and no alignment
  * requirement.  Ranges must not overlap each other.  The device-side offset
  * table built from the arrays is cached inside the library and reused when
- * the same arrays are seen again. */
+ * the same arrays are seen again (one table per distinct set of copies, as many
+ * as the job cycles through); the first call with a new set stages its table with
+ * an asynchronous copy on the same stream and does not wait for the device.
+ * A stream that these entry points have used must be idle when it is destroyed
+ * (hvdhip_stream_destroy sees to that itself). */
 int hvdhip_batched_d2d_memcpy(void* const* out, const void* const* in, const size_t* sizes,
                               int num_copies, void* stream);
+
+/* Counters of the current device's cache of copy tables, for tests: calls that found their
+ * table, calls that built one, tables evicted, tables held now.  Any pointer may be NULL. */
+int hvdhip_copy_cache_stats(uint64_t* hits, uint64_t* misses, uint64_t* evictions, uint64_t* entries);
+/* Limits of the current device's cache of copy tables: at most max_entries tables (at least 1)
+ * and max_bytes of device memory for them; the least recently used go first.  The defaults
+ * (4096 tables, 256 MiB) hold every fusion cycle of a multi-billion-parameter step; this call
+ * exists so that tests can make eviction happen. */
+int hvdhip_copy_cache_set_limits(uint64_t max_entries, uint64_t max_bytes);
 
 /* BatchedScaledD2DMemcpyCudaImpl (ops/cuda/cuda_kernels.h:42, cuda_kernels.cu:289-321):
  * the same copies with every element multiplied by scale_factor.  Arithmetic

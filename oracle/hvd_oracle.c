@@ -499,20 +499,29 @@ static void scaled_add_half(int len, double ca, uint16_t* a, double cb, const ui
   }
 }
 
+/* Keeps the compiler from contracting a product into the sum that follows it
+ * (-mfma with the GNU fp-contract default would): the value passes through a
+ * register untouched. */
+static inline double rounded(double x) {
+  __asm__("" : "+x"(x));
+  return x;
+}
+
 /* Adasum::ScaledAdd<T>, ops/adasum/adasum.h:429-435: a = ca*a + cb*b with the
  * operands promoted to double and the result converted to T; fp16 variant
- * :482-500.  Dispatch as in DispatchScaledAdd, adasum.h:124-140.  The
- * compiler may contract the double expression into an fma, as the reference
- * build (-mfma, GNU fp-contract default) may. */
+ * :482-500.  Dispatch as in DispatchScaledAdd, adasum.h:124-140.  The double
+ * expression is evaluated as the source states it: two rounded products and
+ * their rounded sum.  (A reference build with -mfma may contract one product
+ * into the sum, which moves a result by at most one unit in the last place.) */
 int orc_adasum_scaled_add(int dtype, int count, double ca, void* a, double cb, const void* b) {
   if (dtype == ORC_FLOAT32) {
     float* x = (float*)a;
     const float* y = (const float*)b;
-    for (int i = 0; i < count; ++i) x[i] = (float)(ca * x[i] + cb * y[i]);
+    for (int i = 0; i < count; ++i) x[i] = (float)(rounded(ca * x[i]) + rounded(cb * y[i]));
   } else if (dtype == ORC_FLOAT64) {
     double* x = (double*)a;
     const double* y = (const double*)b;
-    for (int i = 0; i < count; ++i) x[i] = ca * x[i] + cb * y[i];
+    for (int i = 0; i < count; ++i) x[i] = rounded(ca * x[i]) + rounded(cb * y[i]);
   } else if (dtype == ORC_FLOAT16) {
     scaled_add_half(count, ca, (uint16_t*)a, cb, (const uint16_t*)b);
   } else {

@@ -64,12 +64,22 @@ def test_combine_matches_oracle(gpu, orc, dtype):
             # fp16: float coefficients (identical after rounding 1e-13-close doubles, barring a tie) and
             # exact fp32 mul + fma: bit-exact
             assert np.array_equal(got, want)
-        elif dtype == F32:
-            assert _ulp_diff(got, want).max() <= 1
         else:
-            # fp64 results see the 1e-13 coefficient difference (summation order) directly
-            bound = 1e-11 * (np.abs(a.astype(np.float64)) + np.abs(b.astype(np.float64)))
-            assert np.all(np.abs(got - want) <= bound)
+            # The scaled add itself is pinned to the bit: with the coefficients the device computed,
+            # the result is acoeff * a + bcoeff * b as adasum.h:429-435 states it (two rounded double
+            # products, their rounded sum, one conversion), which numpy evaluates without contraction.
+            off = 0
+            for i, c in enumerate(COUNTS):
+                x, y = a[off:off + c].astype(np.float64), b[off:off + c].astype(np.float64)
+                exact = (np.float64(co[2 * i]) * x + np.float64(co[2 * i + 1]) * y).astype(np_t)
+                assert np.array_equal(got[off:off + c].view(np.uint8), exact.view(np.uint8)), i
+                off += c
+            # Against the oracle's own coefficients (sequential sums; 1e-13 apart from the tree sums):
+            if dtype == F32:
+                assert _ulp_diff(got, want).max() <= 1
+            else:
+                bound = 1e-11 * (np.abs(a.astype(np.float64)) + np.abs(b.astype(np.float64)))
+                assert np.all(np.abs(got - want) <= bound)
     finally:
         plan.destroy()
 
@@ -128,6 +138,56 @@ def test_dispatch_hooks_single_layer(gpu, orc):
         assert got[n] == 0
         if n:
             assert _ulp_diff(got[:n], want).max() <= 1
+
+
+def test_dispatch_hooks_from_two_threads_on_two_streams(gpu, orc):
+    # The per-layer hooks keep their single-layer plans in a shared cache.  Two threads, each with
+    # a stream of its own and the same layer sizes, must neither wait for each other's blocking
+    # read nor see each other's partial sums.
+    import ctypes
+    import threading
+    import horovod_amd
+    L = horovod_amd.lib()
+    rng = np.random.default_rng(31)
+    sizes = [70001, 1000, 70001, 333333, 1000]
+    data = []
+    for t in range(2):
+        per = []
+        for n in sizes:
+            a, b = _pair(rng, n, np.float32, corr=0.2 + 0.5 * t)
+            per.append((a, b, gpu.upload(a), gpu.upload(b)))
+        data.append(per)
+    errors, results = [], [[], []]
+
+    def worker(t):
+        try:
+            L.hvdhip_set_device(0)
+            st = horovod_amd.Stream()
+            for rep in range(6):
+                for a, b, d_a, d_b in data[t]:
+                    dot, an, bn = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+                    horovod_amd.check(L.hvdhip_adasum_dot_and_norm_sqrds(
+                        d_a.data_ptr(), d_b.data_ptr(), F32, a.size, ctypes.byref(dot), ctypes.byref(an),
+                        ctypes.byref(bn), st.handle), "dot")
+                    results[t].append((a.size, dot.value, an.value, bn.value))
+            st.destroy()
+        except Exception as e:  # pragma: no cover
+            errors.append(e)
+
+    ts = [threading.Thread(target=worker, args=(t,)) for t in range(2)]
+    [t.start() for t in ts]
+    [t.join() for t in ts]
+    assert not errors, errors
+    for t in range(2):
+        assert len(results[t]) == 6 * len(sizes)
+        for k, (n, dot, an, bn) in enumerate(results[t]):
+            a, b, _, _ = data[t][k % len(sizes)]
+            w = orc.adasum_dot_norms(a, b, F32)
+            assert np.allclose([dot, an, bn], w, rtol=1e-12, atol=0), (t, k)
+        # the same layer gives the same bits every time (fixed summation tree)
+        firsts = {}
+        for k, r in enumerate(results[t]):
+            assert firsts.setdefault(k % len(sizes), r) == r
 
 
 def test_tiny_norms_keep_coefficient_one(gpu, orc):

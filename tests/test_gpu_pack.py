@@ -244,10 +244,71 @@ def test_batched_scaled_d2d_memcpy(gpu, orc, dtype, scale):
         assert np.array_equal(out[o:o + c * es], want.view(np.uint8))
 
 
+def _cache_stats():
+    import ctypes
+    import horovod_amd
+    v = [ctypes.c_uint64() for _ in range(4)]
+    horovod_amd.check(horovod_amd.lib().hvdhip_copy_cache_stats(*[ctypes.byref(x) for x in v]), "stats")
+    return dict(zip(("hits", "misses", "evictions", "entries"), [x.value for x in v]))
+
+
+def _cache_limits(entries, nbytes):
+    import horovod_amd
+    horovod_amd.check(horovod_amd.lib().hvdhip_copy_cache_set_limits(entries, nbytes), "set_limits")
+
+
+def test_batched_copy_tables_stay_resident_over_a_gpt2_sized_step(gpu):
+    """A GPT-2 XL step has 49 fusion cycles, each with a copy set in and a copy set out: 98 distinct
+    (out, in, sizes) sets through the array-taking entry points, alternating over two streams.  Every
+    set builds its table in the first step and finds it in every later one; nothing is evicted."""
+    import horovod_amd
+    rng = np.random.default_rng(21)
+    nsets, per = 98, 12
+    src = Arena(24 << 20)
+    dst = Arena(24 << 20, fill=0x5A)
+    sets = []
+    for _ in range(nsets):
+        sizes = [4 * int(x) for x in rng.integers(1, 4000, per)]
+        so = [src.alloc(n, align=16) for n in sizes]
+        do = [dst.alloc(n, align=16) for n in sizes]
+        for o, n in zip(so, sizes):
+            src.host[o:o + n] = rng.integers(0, 256, n, dtype=np.uint8)
+        sets.append((None, so, do, sizes))
+    src.upload(), dst.upload()
+    streams = [horovod_amd.Stream(), horovod_amd.Stream()]
+    before = _cache_stats()
+    after_step = []
+    for step in range(3):
+        for i, (_, so, do, sizes) in enumerate(sets):
+            st = streams[i % 2]
+            if i % 3 == 0:  # a third of the sets go through the scaled entry point
+                gpu.H.batched_scaled_d2d_memcpy([dst.ptr(o) for o in do], [src.ptr(o) for o in so], sizes, 1.0,
+                                                F32, st)
+            else:
+                gpu.H.batched_d2d_memcpy([dst.ptr(o) for o in do], [src.ptr(o) for o in so], sizes, st)
+        after_step.append(_cache_stats())
+    for st in streams:
+        st.synchronize()
+    assert after_step[0]["misses"] - before["misses"] == nsets
+    assert after_step[1]["misses"] == after_step[0]["misses"], "tables were rebuilt in the second step"
+    assert after_step[2]["misses"] == after_step[0]["misses"], "tables were rebuilt in the third step"
+    assert after_step[2]["hits"] - after_step[0]["hits"] == 2 * nsets
+    assert after_step[2]["evictions"] == before["evictions"]
+    out = dst.download()
+    for _, so, do, sizes in sets:
+        for s_, d_, n in zip(so, do, sizes):
+            assert np.array_equal(out[d_:d_ + n], src.host[s_:s_ + n])
+    for st in streams:
+        st.destroy()
+
+
 def test_batched_copy_cache_eviction_from_several_threads(gpu):
-    # more distinct copy sets than the table cache holds (64), issued from four threads on four streams
+    # more distinct copy sets than the table cache may hold (limited to 64 here), issued from four
+    # threads on four streams: tables are evicted and their buffers reused while launches are in flight
     import threading
     import horovod_amd
+    _cache_limits(64, 256 << 20)
+    evicted_before = _cache_stats()["evictions"]
     rng = np.random.default_rng(12)
     nsets, per = 40, 6
     src = Arena(4 << 20)
@@ -278,7 +339,40 @@ def test_batched_copy_cache_eviction_from_several_threads(gpu):
     ts = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
     [t.start() for t in ts]
     [t.join() for t in ts]
+    stats = _cache_stats()
+    _cache_limits(4096, 256 << 20)
     assert not errors, errors
+    assert stats["evictions"] - evicted_before >= 4 * nsets - 64 and stats["entries"] <= 64
+    out = dst.download()
+    for so, do, sizes in sets:
+        for s_, d_, n in zip(so, do, sizes):
+            assert np.array_equal(out[d_:d_ + n], src.host[s_:s_ + n])
+
+
+def test_batched_copy_cache_bounded_by_bytes(gpu):
+    # the limit that matters is the device memory the tables take: with room for three 4 KiB tables,
+    # five sets evict, and every copy is still right
+    rng = np.random.default_rng(14)
+    _cache_limits(4096, 3 * 4096)
+    before = _cache_stats()
+    src = Arena(1 << 20)
+    dst = Arena(1 << 20, fill=0x5A)
+    sets = []
+    for _ in range(5):
+        sizes = [int(x) for x in rng.integers(1, 5000, 9)]
+        so = [src.alloc(n, align=16) for n in sizes]
+        do = [dst.alloc(n, align=16) for n in sizes]
+        for o, n in zip(so, sizes):
+            src.host[o:o + n] = rng.integers(0, 256, n, dtype=np.uint8)
+        sets.append((so, do, sizes))
+    src.upload(), dst.upload()
+    for rep in range(2):
+        for so, do, sizes in sets:
+            gpu.H.batched_d2d_memcpy([dst.ptr(o) for o in do], [src.ptr(o) for o in so], sizes, gpu.stream)
+    gpu.sync()
+    stats = _cache_stats()
+    _cache_limits(4096, 256 << 20)
+    assert stats["entries"] <= 3 and stats["evictions"] - before["evictions"] >= 7
     out = dst.download()
     for so, do, sizes in sets:
         for s_, d_, n in zip(so, do, sizes):

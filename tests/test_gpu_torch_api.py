@@ -113,6 +113,22 @@ def test_horovod_allreduce_prescale(hvd, gpu, size, half_factor_mode):
         assert torch.equal(summed.cpu(), multiplied), (dtype, dim)
 
 
+@pytest.mark.parametrize("size", [2, 4])
+def test_inplace_allreduce_with_prescale_on_a_single_tensor(hvd, size):
+    """An in-place request travels alone (no fusion buffer): the other ranks' buffers are made from
+    the same tensor and must see it before rank 0 scales it in place."""
+    hvd.init(size=size)
+    torch.manual_seed(7)
+    base = torch.FloatTensor(17, 17).random_(-100, 100).cuda()
+    for fn in ("allreduce_", "allreduce_async_"):
+        t = base.clone()
+        r = getattr(hvd, fn)(t, op=hvd.Sum, prescale_factor=0.5)
+        if fn.endswith("async_"):
+            r = hvd.synchronize(r)
+        assert r.data_ptr() == t.data_ptr()
+        assert torch.equal(t.cpu(), (base * 0.5 * size).cpu()), fn
+
+
 @pytest.mark.parametrize("half_factor_mode", [False, True])
 @pytest.mark.parametrize("size", [1, 2])
 def test_horovod_allreduce_postscale(hvd, gpu, size, half_factor_mode):

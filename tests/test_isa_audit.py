@@ -93,8 +93,8 @@ def test_streaming_stores_carry_one_of_the_two_policies(kernels):
     stores (sc0 sc1); a plain store would leave its lines in L2 for neither reader."""
     checked = 0
     for name, lines in kernels.items():
-        if "finalize_k" in name:
-            continue  # stores a layer's sums and coefficients, nothing streamed
+        if "finalize_k" in name or "one_layer_tables_k" in name:
+            continue  # stores a layer's sums and coefficients, or a chunk table: nothing streamed
         streams_halves = "PackF32F16" in name  # the narrowing pack stores 8 bytes per lane
         # sums and coefficients of a layer or chunk, written by one lane
         small_results = 4 if ("scaled_add_k" in name or "dot_partials_k" in name) else 0
@@ -109,3 +109,21 @@ def test_streaming_stores_carry_one_of_the_two_policies(kernels):
                 assert " sc0 sc1" in ins and " nt" not in ins, (name, ins)
         assert plain <= small_results, (name, plain)
     assert checked > 500, checked
+
+
+def test_scaled_add_products_are_not_fused_into_the_sum(kernels):
+    """ScaledAdd (ops/adasum/adasum.h:429-435) is two rounded double products and their rounded
+    sum.  In the kernels that take their coefficients ready-made the only double arithmetic is
+    that expression, so a fused multiply-add there would be a contracted product."""
+    checked = 0
+    for name, lines in kernels.items():
+        m = re.search(r"scaled_add_kI([fd])Lb0ELb[01]EEE", name)
+        if not m:
+            continue
+        ops = [ins.split()[0] for ins in lines]
+        assert not any(op.startswith(("v_fma_f64", "v_fmac_f64")) for op in ops), name
+        muls = sum(op.startswith("v_mul_f64") for op in ops)
+        adds = sum(op.startswith("v_add_f64") for op in ops)
+        assert muls == 2 * adds and adds > 0, (name, muls, adds)
+        checked += 1
+    assert checked == 4

@@ -80,6 +80,31 @@ def test_pairwise_matches_closed_form(orc, dtype, np_t, tol):
         off += c
 
 
+@pytest.mark.parametrize("dtype,np_t", [(F32, np.float32), (F64, np.float64)])
+def test_scaled_add_is_two_products_and_a_sum(orc, dtype, np_t):
+    # adasum.h:429-435 as written: acoeff * a[i] + bcoeff * b[i] in double, three roundings, then the
+    # conversion to T.  numpy evaluates each operation on its own (no contraction), so a fused
+    # multiply-add in the oracle would show here as last-bit differences.
+    rng = np.random.default_rng(17)
+    for n in (1, 7, 100003):
+        a = rng.standard_normal(n).astype(np_t)
+        b = rng.standard_normal(n).astype(np_t)
+        ca, cb = 0.8312345678901234, 0.9123456789012345
+        want = (np.float64(ca) * a.astype(np.float64) + np.float64(cb) * b.astype(np.float64)).astype(np_t)
+        got = orc.adasum_scaled_add(a, b, ca, cb, dtype)
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    # a contracted evaluation, fma(ca, a, cb*b), computed exactly with rationals, differs from the
+    # above on some of these inputs: the check can tell the two apart
+    from fractions import Fraction
+    a = rng.standard_normal(3000)
+    b = rng.standard_normal(3000)
+    plain = np.float64(ca) * a + np.float64(cb) * b
+    fused = np.array([float(Fraction(ca) * Fraction(float(x)) + Fraction(float(np.float64(cb) * y)))
+                      for x, y in zip(a, b)])
+    assert 0 < np.count_nonzero(plain != fused) < 1500
+    assert np.array_equal(orc.adasum_scaled_add(a, b, ca, cb, F64), plain)
+
+
 def test_fp16_scaled_add_formula(orc):
     # adasum.h:482-500: float coefficients, t = ca*a rounded to fp32, fma(cb, b, t), RNE to half
     rng = np.random.default_rng(13)
