@@ -81,6 +81,7 @@ _PROTOTYPES = {
     "hvdhip_adasum_dot_and_norm_sqrds": (c_int, [c_void_p, c_void_p, c_int, c_int, POINTER(c_double),
                                                  POINTER(c_double), POINTER(c_double), c_void_p]),
     "hvdhip_adasum_dispatch_scaled_add": (c_int, [c_int, c_int, c_double, c_void_p, c_double, c_void_p, c_void_p]),
+    "hvdhip_adasum_combine_static": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),
 }
 
 _lib = None

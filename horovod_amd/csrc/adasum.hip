@@ -318,6 +318,32 @@ __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ ch
   if (t < n) pa[t] = Axpby<T>::f(ca, pa[t], cb, pb[t]);
 }
 
+// Writes the chunk and layer tables of a single layer of `count` elements, as
+// hvdhip_adasum_plan_create lays them out for one layer: chunk c starts at element
+// c * chunk_units and sits at table position xcd_slot(c).
+__global__ __launch_bounds__(kWG) void one_layer_tables_k(Chunk* __restrict__ chunks,
+                                                          Layer* __restrict__ layer, uint32_t nchunks,
+                                                          uint64_t count, uint32_t chunk_units,
+                                                          uint32_t run) {
+  const uint32_t c = blockIdx.x * kWG + threadIdx.x;
+  if (c == 0) *layer = Layer{0, nchunks};
+  if (c >= nchunks) return;
+  const uint64_t start = (uint64_t)c * chunk_units;
+  const uint64_t left = count - start;
+  chunks[xcd_slot(c, nchunks, run)] =
+      Chunk{start, 0, (uint64_t)c, (uint32_t)(left < chunk_units ? left : chunk_units), 0};
+}
+
+// Scratch of hvdhip_adasum_combine_static: the tables and partial sums that a plan would hold in
+// memory it allocates.  One copy per device, for the life of the process.
+constexpr uint32_t kStaticMaxChunks = 16384;  // 256 MiB per vector at 16 KiB per chunk
+constexpr size_t kStaticChunksOff = 0;
+constexpr size_t kStaticPartialsOff = kStaticChunksOff + (size_t)kStaticMaxChunks * sizeof(Chunk);
+constexpr size_t kStaticResultsOff = kStaticPartialsOff + (size_t)kStaticMaxChunks * 3 * sizeof(double);
+constexpr size_t kStaticLayerOff = kStaticResultsOff + 8 * sizeof(double);  // {dot, |a|^2, |b|^2, ca, cb}, padded
+constexpr size_t kStaticScratchBytes = (kStaticLayerOff + sizeof(Layer) + 255) / 256 * 256;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 }  // namespace
 }  // namespace hvdhip
 
@@ -667,6 +693,77 @@ int hvdhip_adasum_dispatch_scaled_add(int dtype, int count, double acoeff, void*
   rc = check_vectors(e->plan, a, b);
   if (rc == 0) rc = plan_scaled_add(e->plan, a, b, nullptr, acoeff, bcoeff, static_cast<hipStream_t>(stream));
   unpin(e);
+  return rc ? rc : ok();
+}
+
+// ---- the combine that allocates nothing -------------------------------------
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+unsigned char* g_scratch_ptr[kMaxDevices];  // the device address of `scratch`, per device
+
+// The address of the current device's copy of `scratch`.  In host code the array's name is only
+// a handle for the symbol; every use below goes through this pointer.
+int static_scratch(unsigned char** out) {
+  int device = 0;
+  HVDHIP_CHECK(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices)
+    return fail(HVDHIP_ERR_INVALID_ARGUMENT, "device %d is beyond the %d devices this entry point serves", device,
+                kMaxDevices);
+  std::lock_guard<std::mutex> g(g_scratch_mu);
+  if (!g_scratch_ptr[device]) {
+    void* p = nullptr;
+    HVDHIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "hipGetSymbolAddress returned no address for the scratch array");
+    g_scratch_ptr[device] = static_cast<unsigned char*>(p);
+  }
+  *out = g_scratch_ptr[device];
+  return 0;
+}
+}  // namespace
+
+int hvdhip_adasum_combine_static(void* a, const void* b, int dtype, int count, double* results,
+                                 void* stream) {
+  if (count < 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "count is negative");
+  if (dtype != HVDHIP_FLOAT16 && dtype != HVDHIP_FLOAT32 && dtype != HVDHIP_FLOAT64)
+    return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE, "Adasum supports FLOAT16, FLOAT32 and FLOAT64, not dtype %d", dtype);
+  if ((uintptr_t)results % sizeof(double)) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "results is not aligned for doubles");
+  const uint32_t chunk_units = chunk_bytes(Family::kAdasum) / (uint32_t)dtype_size(dtype);
+  const uint64_t nchunks = ((uint64_t)count + chunk_units - 1) / chunk_units;
+  if (nchunks > kStaticMaxChunks)
+    return fail(HVDHIP_ERR_TOO_LARGE,
+                "count %d needs %llu chunks of %u elements; hvdhip_adasum_combine_static holds %u (use a plan)",
+                count, (unsigned long long)nchunks, chunk_units, kStaticMaxChunks);
+  unsigned char* base = nullptr;
+  int rc = static_scratch(&base);
+  if (rc) return rc;
+  // A plan-shaped view of the scratch: nothing here is owned, nothing is freed.
+  hvdhip_adasum_plan view;
+  view.nlayers = 1;
+  view.dtype = dtype;
+  view.total = count;
+  view.max_layer_chunks = (uint32_t)nchunks;
+  view.tables.chunks = reinterpret_cast<Chunk*>(base + kStaticChunksOff);
+  view.tables.nchunks = (uint32_t)nchunks;
+  view.partials = reinterpret_cast<double*>(base + kStaticPartialsOff);
+  view.normdots = results ? results : reinterpret_cast<double*>(base + kStaticResultsOff);
+  view.coeffs = view.normdots + 3;
+  view.layers = reinterpret_cast<Layer*>(base + kStaticLayerOff);
+  rc = check_vectors(&view, a, b);
+  if (rc) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // The array keeps what the last call left: the tables are rewritten for this count, and every
+  // partial sum that is read is written first by this call's first pass.
+  const uint32_t run = xcd_run(nchunks, chunk_bytes(Family::kAdasum), true);
+  launch(one_layer_tables_k, (uint32_t)(nchunks / kWG + 1), s, view.tables.chunks, view.layers,
+         (uint32_t)nchunks, (uint64_t)count, chunk_units, run);
+  HVDHIP_CHECK_LAUNCH("one_layer_tables_k");
+  const bool fused = fused_coeffs(&view);
+  rc = plan_dot_norms(&view, a, b, s, !fused);
+  if (rc) return rc;
+  rc = fused ? scaled_add_by_dtype<true>(&view, a, b, nullptr, 0., 0., s)
+             : plan_scaled_add(&view, a, b, view.coeffs, 0., 0., s);
   return rc ? rc : ok();
 }
 

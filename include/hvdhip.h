@@ -335,6 +335,26 @@ int hvdhip_adasum_dot_and_norm_sqrds(const void* a, const void* b, int dtype, in
 int hvdhip_adasum_dispatch_scaled_add(int dtype, int count, double acoeff, void* a,
                                       double bcoeff, const void* b, void* stream);
 
+/* hvdhip_adasum_combine for a single layer of count elements, for callers that cannot
+ * allocate.  It has no counterpart in the reference: it exists for code under HIP graph
+ * capture, tight serving loops and harnesses that forbid hipMalloc, which cannot create the
+ * plan (device tables, partial sums) that hvdhip_adasum_combine works from.  The tables and
+ * partial sums live in a fixed array of about 0.9 MiB inside the library's device code instead;
+ * every device the library runs on holds its copy until the process ends.  The call only
+ * launches kernels: no allocation, no free, no copy, no fill, no synchronisation.  (The first
+ * call on a device looks the array's address up, which loads the library's device code if
+ * nothing else has: make one call, count 0 will do, before capturing a graph.)
+ *
+ * a and b are device vectors of count elements of dtype (FLOAT16, FLOAT32, FLOAT64); a is
+ * updated in place exactly as hvdhip_adasum_combine with a one-layer plan would.  results is
+ * NULL or a device pointer to 5 doubles that receive {dot, |a|^2, |b|^2, ca, cb}.
+ * Limit: count may need at most 16,384 chunks of 16 KiB, i.e. 2^26 FLOAT32, 2^27 FLOAT16 or
+ * 2^25 FLOAT64 elements (256 MiB per vector); beyond that HVDHIP_ERR_TOO_LARGE is returned and
+ * nothing is launched.  All calls on one device share the one array: calls that overlap in time
+ * on a device (different streams, or threads) race on it; order them on one stream. */
+int hvdhip_adasum_combine_static(void* a, const void* b, int dtype, int count, double* results,
+                                 void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,101 @@
+"""hvdhip_adasum_combine_static, the Adasum combine that allocates nothing (its tables and
+partial sums live in a fixed array inside the library's device code), against
+hvdhip_adasum_combine with a one-layer plan: same kernels, same tables, so the vector, the sums
+and the coefficients must agree to the bit.  Two calls in a row share the array; the second is
+smaller, so it runs over what the first left behind."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle_util import F16, F32, F64, NP_OF
+
+pytestmark = pytest.mark.gpu
+
+
+def _pair(rng, n, np_t, corr=0.3):
+    a = rng.standard_normal(n)
+    b = corr * a + np.sqrt(1 - corr * corr) * rng.standard_normal(n)
+    return a.astype(np_t), b.astype(np_t)
+
+
+def _static(gpu, d_a, d_b, dtype, n, d_res):
+    import horovod_amd
+    horovod_amd.check(horovod_amd.lib().hvdhip_adasum_combine_static(
+        d_a.data_ptr(), d_b.data_ptr(), dtype, n, d_res.data_ptr() if d_res is not None else None,
+        gpu.stream.handle), "hvdhip_adasum_combine_static")
+
+
+def _planned(gpu, d_a, d_b, dtype, n):
+    plan = gpu.H.AdasumPlan([n], dtype)
+    try:
+        plan.combine(d_a.data_ptr(), d_b.data_ptr(), gpu.stream)
+        nd, co = plan.read(gpu.stream)
+    finally:
+        plan.destroy()
+    return np.array(nd + co)
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, F64])
+def test_two_calls_in_a_row_match_the_planned_combine(gpu, orc, dtype):
+    rng = np.random.default_rng(41)
+    np_t = NP_OF[dtype]
+    raw = np.uint16 if np_t == np.float16 else np_t
+    per_chunk = 16384 // np.dtype(np_t).itemsize
+    # first call: 700 chunks (the sums get a launch of their own) and a ragged tail;
+    # second call: 37 chunks (summed inside the scaled add), over the first call's leftovers;
+    # then the empty layer and a single element
+    for n in (700 * per_chunk + 1234, 37 * per_chunk - 5, 0, 1):
+        a, b = _pair(rng, max(n, 1), np_t)
+        a, b = a[:n], b[:n]
+        guard = np.full(8, 7, np_t)
+        d_a1 = gpu.upload(np.concatenate([a, guard]))
+        d_a2 = gpu.upload(np.concatenate([a, guard]))
+        d_b = gpu.upload(np.concatenate([b, guard]))
+        d_res = torch.full((5,), -1.0, dtype=torch.float64, device="cuda")
+        torch.cuda.synchronize()
+        want5 = _planned(gpu, d_a1, d_b, dtype, n)
+        _static(gpu, d_a2, d_b, dtype, n, d_res)
+        got = gpu.download(d_a2, raw)
+        want = gpu.download(d_a1, raw)
+        assert np.array_equal(got, want), "vector differs from the planned combine (n=%d)" % n
+        assert np.array_equal(got[n:], guard.view(raw)), "wrote past the vector"
+        got5 = d_res.cpu().numpy()
+        assert np.array_equal(got5.view(np.uint64), want5.view(np.uint64)), (n, got5, want5)
+        if n:
+            # and the planned combine is what the oracle computes (coefficients to 1e-6)
+            _, _, co_w = orc.adasum_pairwise(a.view(raw), b.view(raw), [n], dtype)
+            assert np.all(np.abs(got5[3:] - co_w) <= 1e-6 * np.abs(co_w))
+            assert not np.array_equal(got[:n], a.view(raw)), "the vector was left untouched"
+
+
+def test_results_pointer_is_optional_and_limit_is_enforced(gpu):
+    import horovod_amd
+    rng = np.random.default_rng(42)
+    n = 100000
+    a, b = _pair(rng, n, np.float32)
+    d_a1, d_a2, d_b = gpu.upload(a), gpu.upload(a), gpu.upload(b)
+    _planned(gpu, d_a1, d_b, F32, n)
+    _static(gpu, d_a2, d_b, F32, n, None)
+    assert np.array_equal(gpu.download(d_a2, np.float32), gpu.download(d_a1, np.float32))
+    # one element beyond 16,384 chunks of 4,096 floats: refused, nothing launched
+    with pytest.raises(horovod_amd.HvdHipError) as e:
+        _static(gpu, d_a2, d_b, F32, (1 << 26) + 1, None)
+    assert e.value.code == -4
+    with pytest.raises(horovod_amd.HvdHipError) as e:
+        _static(gpu, d_a2, d_b, 4, 16, None)  # INT32
+    assert e.value.code == -2
+
+
+def test_largest_size_runs(gpu):
+    # exactly the limit for fp32: 2^26 elements, 16,384 chunks; identical vectors give the vector back
+    n = 1 << 26
+    x = torch.ones(n, dtype=torch.float32, device="cuda")
+    y = torch.ones(n, dtype=torch.float32, device="cuda")
+    d_res = torch.zeros(5, dtype=torch.float64, device="cuda")
+    torch.cuda.synchronize()
+    _static(gpu, x, y, F32, n, d_res)
+    gpu.sync()
+    assert d_res.cpu().tolist() == [float(n)] * 3 + [0.5, 0.5]
+    assert int((x != 1).sum()) == 0
