@@ -1,20 +1,28 @@
 #!/usr/bin/env python3
 """Throughput of the fusion-buffer hot path on one MI355X.
 
-One "step" is one pass of the hot path over one batch of synthetic gradients.
-The headline workload is the fusion stress configuration: 1,024 fp32 tensors
-with element counts log-uniform in [256, 65536] (seed 3), values U(-1,1)
-(seed 4), packed into a 64 MiB fusion buffer with prescale 0.125 and unpacked
-again.  Inputs are resident in HBM before the timed region starts.
+The headline workload is the pipeline the metric names, on the ResNet-50 configuration: 161 fp32
+gradient tensors (25,557,032 elements, N(0, 1e-3)), fused by the reference's planner into two
+cycles of at most 64 MiB; per cycle a pack with prescale 0.125 into the fusion buffer, the
+reduce-sum of the buffer with one peer buffer resident on the same device, and the unpack
+(postscale 1.0) -- the sequence of NCCLAllreduce::Execute (ops/nccl_operations.cc:156-214) with
+the collective replaced by the local sum.  One "step" is REPS passes of that pipeline over
+tensor sets that rotate so that no pass finds its inputs in the 256 MB Infinity Cache.  Inputs
+are resident in HBM before the timed region starts; everything runs on one stream.
 
-Prints ONE JSON line.  `value` is algorithmic GB/s of the whole step
-(pack = P_in + P_buf, unpack = P_buf + P_out); `roofline` prices the dominant
-kernel (the scaled pack) against the 8 TB/s HBM peak from its average launch
-duration measured with HIP events on the stream it runs on; `cpu_baseline` is
-the CPU oracle (a restatement of the reference's CPU path) timed on one host
-core over the same workload; `extra` carries the other pipelines (ResNet-50
-cycle with a peer reduce, BERT-large fp16-compressed with 7 peers, Adasum,
-GPT-2 XL streamed on two streams).
+Prints ONE JSON line.  `value` is ALGORITHMIC GB/s of the whole step (pack = P_in + P_buf,
+reduce = (k+2) C, unpack = P_buf + P_out; the bytes a pipeline must move with the fusion buffer
+materialised on both sides of the collective) -- not an HBM counter: inside a cycle the fusion
+buffer is handed from kernel to kernel through the Infinity Cache, so a pipeline's algorithmic
+rate can exceed what any one of its kernels streams out of HBM.  The HBM claim is `roofline`:
+the dominant kernel of the workload launched back to back on rotating buffers, algorithmic bytes
+per launch over its average duration from HIP events on its stream, against the 8 TB/s peak.
+`cpu_baseline` is the CPU oracle (a restatement of the reference's CPU path) on one host core
+over the same workload.  `extra` carries the other configurations, each with the same roofline
+block for every kernel family it launches (`kernels`), the dominant one repeated as `roofline`.
+
+`--kernel-only <config>` runs exactly the back-to-back kernel loops of one configuration and
+nothing else, for rocprofv3 (the summaries under profiles/ come from these runs).
 """
 import argparse
 import json
@@ -29,42 +37,52 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch of the scaled pack kernel on the headline workload, from rocprofv3
-# FETCH_SIZE and WRITE_SIZE runs of `bench.py --kernel-only`, each scaled by what the same
-# counter reads for a plain 256 MiB copy (`bench.py --calibrate`): FETCH_SIZE x 1.9544,
-# WRITE_SIZE x 1.0000.  The summary with the commands is profiles/pack_kernel_fusion_stress.txt.
-PACK_TRAFFIC_BYTES_MEASURED = 93204449
+# One step of the headline = this many passes of the two-cycle ResNet-50 pipeline (a pass takes
+# about 0.11 ms; a step of 50 passes keeps even a short run measuring the device, not the host's
+# wake-up after the final synchronisation).
+REPS = 50
 
+# Independent copies of a configuration's buffers that launches rotate over.
+ROTATE = 6
 
-# One step of the headline is the fusion stress workload as the baseline configuration states it:
-# 200 repetitions of pack + unpack over the 1,024 tensors.
-REPS = 200
+# HBM bytes per launch, per kernel of the --kernel-only loops, from rocprofv3 FETCH_SIZE and
+# WRITE_SIZE runs (KiB per dispatch), each scaled by what the same counter reads for a plain
+# 256 MiB device copy (`bench.py --calibrate`).  The summaries with the commands are the files
+# named here under profiles/; tests/test_host_logic.py re-derives every figure from them.
+TRAFFIC_BYTES_MEASURED = {
+}
+TRAFFIC_PROFILE = {
+    "c1": "profiles/c1_resnet50_fp32_kernels.txt",
+    "c2": "profiles/c2_fusion_stress_kernels.txt",
+    "c3": "profiles/c3_bert_large_fp16_kernels.txt",
+    "c4": "profiles/c4_adasum_fp32_kernels.txt",
+    "c5": "profiles/c5_gpt2_xl_fp16_kernels.txt",
+}
+
+CONFIGS = ("c1", "c2", "c3", "c4", "c5")
 
 
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20,
-                    help="timed steps; one step is the workload's %d repetitions of pack + unpack" % REPS)
+                    help="timed steps; one step is %d passes of the ResNet-50 pipeline" % REPS)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--kernel-only", nargs="?", const="pack", default=None,
-                    choices=["pack", "reduce", "adasum"],
-                    help="only launch one kernel family (for rocprofv3 runs): the scaled pack of the headline "
-                         "workload (default), the fp32 reduce-sum of a 64 MiB buffer with one peer, or the "
-                         "Adasum combine of 2 x 2^25 fp32 in 64 layers")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--kernel-only", choices=CONFIGS + ("c4h",), default=None,
+                    help="only the back-to-back kernel loops of one configuration (for rocprofv3 runs): c1 ResNet-50 "
+                         "fp32 cycle, c2 fusion stress, c3 BERT-large fp32->fp16 cycle with 7 peers on the 1/8 share, "
+                         "c4 Adasum 2 x 2^25 fp32, c4h the same in fp16, c5 GPT-2 XL fp16 cycle and embedding; "
+                         "--steps launches per kernel after --warmup")
     ap.add_argument("--calibrate", action="store_true",
                     help="only launch a plain 256 MiB device copy (scales rocprofv3 byte counters)")
-    ap.add_argument("--streams", type=int, default=2,
-                    help="stream slots the headline steps alternate over, each with a fusion buffer of its own "
-                         "(HOROVOD_NUM_NCCL_STREAMS); default 2, the configuration this library is meant to run "
-                         "in; the one-stream figure is reported beside it")
-    ap.add_argument("--replicas", type=int, default=8,
-                    help="independent copies of the workload that steps rotate over, so that the "
-                         "bytes touched between two uses of one copy exceed the 256 MB Infinity Cache")
     return ap.parse_args()
 
+
+# ----------------------------------------------------------------------------------------------
+# timing
+# ----------------------------------------------------------------------------------------------
 
 def timed(fn, sync, steps, warmup):
     """Wall time of `steps` calls of fn bracketed by synchronisation on both sides."""
@@ -97,6 +115,23 @@ def event_timed(fn, stream, steps, warmup):
     return ms / steps * 1e-3
 
 
+_PAIR = []
+
+
+def stream_pair():
+    """Two library streams created once, before any other, and shared by everything in this run:
+    streams that are created later, while others exist, can land on a hardware queue that is
+    already in use and then overlap nothing."""
+    if not _PAIR:
+        from horovod_amd import Stream
+        _PAIR.extend([Stream(), Stream()])
+    return _PAIR
+
+
+# ----------------------------------------------------------------------------------------------
+# device data
+# ----------------------------------------------------------------------------------------------
+
 class DeviceSet:
     """Gradient tensors carved out of one device allocation at 256-byte aligned offsets."""
 
@@ -115,72 +150,339 @@ class DeviceSet:
         self.ptrs = [self.dev.data_ptr() + o for o in offs]
 
 
-def stress_workload(replicas):
-    """Returns counts, the host image of the tensors, and `replicas` (src, dst) device sets."""
+_GEN = []
+
+
+def randn_bytes(nbytes, dtype, std, seed):
+    """nbytes of N(0, std) values of torch dtype `dtype`, as a uint8 device tensor."""
     import torch
-    from horovod_amd import workloads as W
-    counts = W.stress_counts(seed=3)
-    rng = np.random.default_rng(4)
-    host = np.zeros(sum((c * 4 + 255) // 256 * 256 for c in counts), np.uint8)
-    off = 0
-    for c in counts:
-        host[off:off + 4 * c] = rng.uniform(-1, 1, c).astype(np.float32).view(np.uint8)
-        off += (c * 4 + 255) // 256 * 256
+    if not _GEN:
+        _GEN.append(torch.Generator(device="cuda"))
+    g = _GEN[0]
+    g.manual_seed(seed)
+    n = nbytes // torch.empty(0, dtype=dtype).element_size()
+    return (torch.randn(n, generator=g, device="cuda", dtype=torch.float32) * std).to(dtype).view(torch.uint8)
+
+
+def zeros_bytes(nbytes):
+    import torch
+    return torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+
+
+def torch_dtype(dtype):
+    import torch
+    from horovod_amd import DTYPE
+    return {DTYPE["float32"]: torch.float32, DTYPE["float16"]: torch.float16}[dtype]
+
+
+# ----------------------------------------------------------------------------------------------
+# kernel loops: every kernel family of a configuration, launched back to back on rotating buffers
+# ----------------------------------------------------------------------------------------------
+
+class Case:
+    """One kernel at one grid.  fn() queues one launch on `stream` (the next rotating buffer set
+    every call); alg = algorithmic bytes per launch; kernel = its name as a profiler prints it."""
+
+    def __init__(self, key, kernel, fn, alg, what, workgroups=None, cleanup=None):
+        self.key, self.kernel, self.fn, self.alg, self.what, self.workgroups = key, kernel, fn, alg, what, workgroups
+        self.cleanup = cleanup  # destroys the plans behind fn (the closures hold the device memory)
+
+
+def cycle_cases(cfg, counts, tdtype, bdtype, std, peers, share_world, stream, pack_kernel, reduce_kernel,
+                unpack_kernel, seed0):
+    """Pack, reduce-sum and unpack of ONE fusion cycle, each launched back to back:
+    pack reads another replica's tensors every launch and writes the slot's one fusion buffer (as the
+    reference keeps one per stream slot); the reduce-sum and the unpack rotate over ROTATE buffers."""
+    import torch
+    from horovod_amd import FusionPlan, dtype_size, host as H, workloads as W
+    ts, bs = dtype_size(tdtype), dtype_size(bdtype)
+    tt, bt = torch_dtype(tdtype), torch_dtype(bdtype)
     sets = []
-    for _ in range(replicas):
-        src = DeviceSet(counts, 4, lambda n: torch.from_numpy(host).cuda())
-        dst = DeviceSet(counts, 4, lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
-        sets.append((src, dst))
-    return counts, host, sets
+    for r in range(ROTATE):
+        src = DeviceSet(counts, ts, lambda n: randn_bytes(n, tt, std, seed0 + r))
+        dst = DeviceSet(counts, ts, zeros_bytes)
+        sets.append((src, dst, FusionPlan(src.ptrs, dst.ptrs, counts, tdtype, bdtype)))
+    plan0 = sets[0][2]
+    blen = plan0.buffer_len
+    nelem = blen // bs
+    share = nelem if share_world == 1 else W.reduce_scatter_share(nelem, share_world)
+    slack = 4096 * bs
+    fb_pack = zeros_bytes(blen + slack)
+    fbs = [randn_bytes((blen + slack + 255) // 256 * 256, bt, std, seed0 + 50 + r) for r in range(ROTATE)]
+    peer_bufs = [[randn_bytes((share * bs + 255) // 256 * 256, bt, std, seed0 + 100 + 16 * r + p) for p in range(peers)]
+                 for r in range(ROTATE)]
+    torch.cuda.synchronize()
+    payload = sum(counts)
+    turn = [0]
+
+    def rot():
+        turn[0] = (turn[0] + 1) % ROTATE
+        return turn[0]
+
+    def pack():
+        sets[rot()][2].pack(fb_pack.data_ptr(), 0.125, stream)
+
+    def reduce():
+        i = rot()
+        H.reduce_sum_k(fbs[i].data_ptr(), [p.data_ptr() for p in peer_bufs[i]], share, bdtype, stream)
+
+    def unpack():
+        i = rot()
+        sets[i][2].unpack(fbs[i].data_ptr(), 1.0, stream)
+
+    def cleanup():
+        for _, _, plan in sets:
+            plan.destroy()
+
+    tile = 4096 // bs
+    cases = [
+        Case(cfg + ".pack", pack_kernel, pack, payload * (ts + bs),
+             "pack with prescale 0.125 of %d tensors (%d payload bytes in, %d in the buffer); tensors of another replica "
+             "every launch, the slot's one fusion buffer as destination" % (len(counts), payload * ts, payload * bs),
+             plan0.num_chunks, cleanup),
+        Case(cfg + ".reduce", reduce_kernel, reduce, (peers + 2) * share * bs,
+             "resident chunk of %d bytes += %d peer chunk(s) in one pass; %d (resident, peers) sets rotated"
+             % (share * bs, peers, ROTATE), (share + tile - 1) // tile),
+        Case(cfg + ".unpack", unpack_kernel, unpack, payload * (bs + ts),
+             "unpack (postscale 1.0) of the same tensors; fusion buffer and outputs of another replica every launch"),
+    ]
+    return cases
 
 
-def cpu_baseline_stress(counts, host, budget_s=12.0):
-    """The reference CPU sequence (ops/gloo_operations.cc:118-170) on one core:
-    memcpy pack, in-place ScaleBuffer(0.125), memcpy unpack."""
+def build_cases(cfg):
+    """The kernel loops of one configuration (all on the first stream of the pair)."""
+    import torch
+    from horovod_amd import AdasumPlan, DTYPE, FusionPlan, host as H, workloads as W
+    F32, F16 = DTYPE["float32"], DTYPE["float16"]
+    s = stream_pair()[0]
+    if cfg == "c1":
+        counts = [W.numel(x) for x in W.resnet50_shapes()]
+        g0 = W.fuse([4 * c for c in counts])[0]
+        return cycle_cases("c1", [counts[i] for i in g0], F32, F32, 1e-3, 1, 1, s,
+                           "xfer_k<Scale<float, float>, 0, true>", "reduce_k<float, 1, true>",
+                           "xfer_k<Copy<unsigned int>, 1, false>", 1000)
+    if cfg == "c2":
+        counts = W.stress_counts(seed=3)
+        cases = cycle_cases("c2", counts, F32, F32, 1.0, 1, 1, s, "xfer_k<Scale<float, float>, 0, true>",
+                            "reduce_k<float, 1, true>", "xfer_k<Copy<unsigned int>, 1, false>", 2000)
+        return [cases[0], cases[2]]  # the stress configuration has no reduce stage
+    if cfg == "c3":
+        counts = [W.numel(x) for x in W.bert_large_shapes()]
+        g1 = W.fuse([2 * c for c in counts])[1]
+        return cycle_cases("c3", [counts[i] for i in g1], F32, F16, 1e-4, 7, 8, s,
+                           "xfer_k<PackF32F16, 0, true>", "reduce_k<_Float16, 7, true>",
+                           "xfer_k<UnpackF16F32, 1, false>", 3000)
+    if cfg == "c5":
+        counts = [W.numel(x) for x in W.gpt2_xl_shapes()]
+        groups = W.fuse([2 * c for c in counts])
+        layer = next(g for g in groups if len(g) == 12)
+        cases = cycle_cases("c5", [counts[i] for i in layer], F16, F16, 1e-3, 1, 1, s,
+                            "xfer_k<ScaleHalf, 0, true>", "reduce_k<_Float16, 1, true>",
+                            "xfer_k<Copy<unsigned short>, 1, false>", 5000)
+        # the 50257 x 1600 embedding exceeds the threshold and travels alone: prescale tensor -> output,
+        # sum in place (ops/nccl_operations.cc:176-186)
+        n = counts[0]
+        emb = [(randn_bytes(2 * n, torch.float16, 1e-3, 5100 + r), zeros_bytes(2 * n),
+                randn_bytes(2 * n, torch.float16, 1e-3, 5200 + r)) for r in range(3)]
+        torch.cuda.synchronize()
+        turn = [0]
+
+        def scale():
+            i = turn[0] = (turn[0] + 1) % len(emb)
+            H.scale_buffer(emb[i][0].data_ptr(), emb[i][1].data_ptr(), n, 0.125, F16, s)
+
+        def reduce_emb():
+            i = turn[0] = (turn[0] + 1) % len(emb)
+            H.reduce_sum(emb[i][1].data_ptr(), emb[i][2].data_ptr(), n, F16, s)
+
+        cases += [
+            Case("c5.scale_single", "contig_k<ScaleHalf, false>", scale, 4 * n,
+                 "the embedding (%d halves) scaled by 0.125 from tensor to output; 3 pairs rotated" % n,
+                 (2 * n + 4095) // 4096),
+            Case("c5.reduce_single", "reduce_k<_Float16, 1, true>", reduce_emb, 6 * n,
+                 "the embedding summed in place with one peer; 3 pairs rotated", (2 * n + 4095) // 4096),
+        ]
+        return cases
+    if cfg in ("c4", "c4h"):
+        n = 1 << 25
+        dt, tdt, es = (F32, torch.float32, 4) if cfg == "c4" else (F16, torch.float16, 2)
+        tname = "float" if cfg == "c4" else "_Float16"
+        lc = W.adasum_layer_counts(n, 64, seed=13)
+        g = torch.Generator(device="cuda")
+        pairs = []
+        for r in range(4):
+            g.manual_seed(14 + 2 * r)
+            a = torch.randn(n, generator=g, device="cuda", dtype=torch.float32)
+            g.manual_seed(15 + 2 * r)
+            b = 0.3 * a + (1 - 0.09) ** 0.5 * torch.randn(n, generator=g, device="cuda", dtype=torch.float32)
+            pairs.append((a.to(tdt), b.to(tdt)))
+        plan = AdasumPlan(lc, dt)
+        torch.cuda.synchronize()
+        turn = [0]
+
+        def combine():
+            # the combine rewrites a; its cost does not depend on the values, which stay finite
+            i = turn[0] = (turn[0] + 1) % len(pairs)
+            plan.combine(pairs[i][0].data_ptr(), pairs[i][1].data_ptr(), s)
+
+        return [Case(cfg + ".combine", "dot_partials_k<%s, true> + scaled_add_k<%s, true, false>" % (tname, tname),
+                     combine, 5 * n * es,
+                     "Adasum combine of two vectors of 2^25 elements in 64 layers: first pass 2 N s bytes (keeps the pair "
+                     "in the Infinity Cache), second pass 3 N s bytes; 4 pairs rotated", None, plan.destroy)]
+    raise ValueError(cfg)
+
+
+def measure_cases(cases, steps=100, warmup=10):
+    """Roofline block per case, from HIP events on the stream the kernel is launched on."""
+    s = stream_pair()[0]
+    out = []
+    for c in cases:
+        sec = event_timed(c.fn, s, steps, warmup)
+        gbs = c.alg / sec / 1e9
+        out.append({"bound": "hbm", "kernel": c.kernel, "case": c.key, "launch_us": round(sec * 1e6, 2),
+                    "algorithmic_bytes_per_launch": c.alg, "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                    "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                    "traffic": TRAFFIC_BYTES_MEASURED.get(c.key), "workgroups": c.workgroups, "timed": c.what})
+    return out
+
+
+def release(cases):
+    """Destroys the plans of the cases and lets go of their device memory."""
+    import torch
+    torch.cuda.synchronize()
+    for c in cases:
+        if c.cleanup:
+            c.cleanup()
+        c.cleanup = c.fn = None
+    torch.cuda.empty_cache()
+
+
+# ----------------------------------------------------------------------------------------------
+# whole pipelines
+# ----------------------------------------------------------------------------------------------
+
+class PipelineRun:
+    """A configuration's whole pipeline over `replicas` rotating tensor sets.  All replicas queue on
+    the same stream(s) and share the one fusion buffer of each stream slot."""
+
+    def __init__(self, shapes, tdtype, bdtype, std, peers, fraction, streams, replicas, arrays=False):
+        import torch
+        from horovod_amd import dtype_size, workloads as W
+        from horovod_amd.pipeline import AllreducePipeline
+        es = dtype_size(tdtype)
+        self.counts = [W.numel(x) for x in shapes]
+        self.peers, self.fraction = peers, fraction
+        self.reps = []
+        shared = stream_pair()[:streams]
+        buffers = None
+        for r in range(replicas):
+            src = DeviceSet(self.counts, es, lambda n: randn_bytes(n, torch_dtype(tdtype), std, 1 + r))
+            dst = DeviceSet(self.counts, es, zeros_bytes)
+            pipe = AllreducePipeline(src.ptrs, dst.ptrs, self.counts, tdtype, bdtype, streams=shared, buffers=buffers,
+                                     array_entry_points=arrays)
+            buffers = pipe.buffers
+            bs = dtype_size(pipe.buffer_dtype)
+            # one buffer per peer, sized for the largest cycle's reduced chunk, serves every cycle
+            need = max(pipe.reduce_elems(c, fraction) for c in pipe.cycles) * bs
+            peer_bufs = [randn_bytes((need + 255) // 256 * 256, torch_dtype(pipe.buffer_dtype), std, 100 + 16 * r + p)
+                         for p in range(peers)]
+            self.reps.append((src, dst, pipe, peer_bufs))
+        torch.cuda.synchronize()
+        self.turn = 0
+        self.pipe = self.reps[0][2]
+
+    def one_pass(self):
+        self.turn += 1
+        _, _, pipe, peer_bufs = self.reps[self.turn % len(self.reps)]
+        # a single-cycle configuration alternates its passes over the stream slots
+        first_slot = self.turn if len(pipe.cycles) == 1 else 0
+        pipe.run(0.125, 1.0, (lambda ci, p: peer_bufs[p].data_ptr()) if self.peers else None, self.peers,
+                 self.fraction, True, first_slot=first_slot)
+
+    def sync(self):
+        for _, _, pipe, _ in self.reps:
+            pipe.synchronize()
+
+    def algorithmic_bytes(self):
+        return self.pipe.algorithmic_bytes(self.peers, self.fraction, True)
+
+    def destroy(self):
+        import torch
+        for _, _, pipe, _ in self.reps:
+            pipe.destroy()
+        self.reps = []
+        torch.cuda.empty_cache()
+
+
+def pipeline_figures(run, sec, streams, note=None):
+    ab = run.algorithmic_bytes()
+    d = {"algorithmic_GB/s": round(ab / sec / 1e9, 1), "algorithmic_frac_of_8TBps": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4),
+         "ms": round(sec * 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1), "cycles": len(run.pipe.cycles),
+         "streams": streams, "peers": run.peers, "reduce": "k-way" if run.peers else None,
+         "completion_event_per_cycle": run.pipe.completion_events, "replicas_rotated": len(run.reps)}
+    if note:
+        d["note"] = note
+    return d
+
+
+# ----------------------------------------------------------------------------------------------
+# CPU baselines: the oracle on one host core, same algorithmic bytes
+# ----------------------------------------------------------------------------------------------
+
+def _oracle():
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle_util
+    return oracle_util, oracle_util.Oracle().lib
+
+
+def cpu_baseline_resnet(budget_s=12.0):
+    """The reference CPU sequence (ops/gloo_operations.cc:118-170) over the whole ResNet-50 set:
+    memcpy pack, in-place ScaleBuffer(0.125), sum with one peer buffer, memcpy unpack (7P bytes)."""
     from ctypes import c_double, c_int, c_int64, c_void_p
-    orc = oracle_util.Oracle()
-    L = orc.lib
-    offs, cur = [], 0
-    for c in counts:
-        offs.append(cur)
-        cur += (c * 4 + 255) // 256 * 256
-    out = np.zeros_like(host)
-    n = len(counts)
-    tptr = (c_void_p * n)(*[host.ctypes.data + o for o in offs])
-    optr = (c_void_p * n)(*[out.ctypes.data + o for o in offs])
+    from horovod_amd import workloads as W
+    ou, L = _oracle()
+    rng = np.random.default_rng(1)
+    counts = [W.numel(s) for s in W.resnet50_shapes()]
+    ts = [(rng.standard_normal(c, dtype=np.float32) * np.float32(1e-3)) for c in counts]
+    outs = [np.empty_like(t) for t in ts]
+    n, k = sum(counts), len(counts)
     nb = np.array([4 * c for c in counts], np.int64)
-    payload = int(nb.sum())
-    buf = np.zeros(payload + 64, np.uint8)
+    buf = np.zeros(n, np.float32)
+    peer = np.random.default_rng(2).standard_normal(n, dtype=np.float32) * np.float32(1e-3)
+    tp = (c_void_p * k)(*[t.ctypes.data for t in ts])
+    op = (c_void_p * k)(*[t.ctypes.data for t in outs])
+    P = lambda a: c_void_p(a.ctypes.data)  # noqa: E731
+
+    def one():
+        L.orc_pack(tp, P(nb), c_int(k), P(buf))
+        L.orc_scale_buffer(P(buf), P(buf), c_int64(n), c_double(0.125), c_int(ou.F32))
+        L.orc_sum(P(peer), P(buf), c_int64(n), c_int(ou.F32))
+        L.orc_unpack(P(buf), op, P(nb), c_int(k))
+
+    one()
     reps, t0 = 0, time.perf_counter()
     while True:
-        L.orc_pack(tptr, c_void_p(nb.ctypes.data), c_int(n), c_void_p(buf.ctypes.data))
-        L.orc_scale_buffer(c_void_p(buf.ctypes.data), c_void_p(buf.ctypes.data), c_int64(payload // 4),
-                           c_double(0.125), c_int(oracle_util.F32))
-        L.orc_unpack(c_void_p(buf.ctypes.data), optr, c_void_p(nb.ctypes.data), c_int(n))
+        one()
         reps += 1
         dt = time.perf_counter() - t0
         if dt > budget_s:
             break
-    gbs = 4 * payload * reps / dt / 1e9
+    gbs = 7 * 4 * n * reps / dt / 1e9
     return {"value": round(gbs, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": "%d repetitions of the same 1,024-tensor workload (memcpy pack, in-place ScaleBuffer 0.125, "
-                      "memcpy unpack; 4P algorithmic bytes each) in %.1f s; host has %d cores"
+            "sample": "%d passes over the whole 161-tensor set (memcpy pack, in-place ScaleBuffer 0.125, sum with one "
+                      "peer buffer, memcpy unpack; 7P algorithmic bytes each, one buffer for all tensors as the CPU "
+                      "path has no 64 MiB cycles to gain from) in %.1f s; host has %d cores"
                       % (reps, dt, os.cpu_count())}
 
 
 def cpu_extras(budget_s=2.5):
-    """The CPU oracle on one core over bounded samples of the other pipelines, in the same
-    algorithmic bytes as the GPU figures: the whole ResNet-50 set, one 42-tensor BERT-large cycle
-    (cast and scale fused into the copy, which flatters the CPU), the whole Adasum pair, one
-    GPT-2 XL layer.  Buffers are preallocated and every oracle call works in place."""
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    import oracle_util
+    """The CPU oracle on one core over bounded samples of the other configurations, in the same
+    algorithmic bytes as the GPU figures: the stress set, one 42-tensor BERT-large cycle (cast and
+    scale fused into the copy, which flatters the CPU), the whole Adasum pair, one GPT-2 XL layer."""
     from ctypes import c_double, c_int, c_int64, c_void_p
-    from oracle_util import F16, F32
     from horovod_amd import workloads as W
-    L = oracle_util.Oracle().lib
+    ou, L = _oracle()
+    F16, F32 = ou.F16, ou.F32
     rng = np.random.default_rng(0)
     out = {}
 
@@ -190,7 +492,7 @@ def cpu_extras(budget_s=2.5):
     def ptrs(arrays):
         return (c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
 
-    def run(name, fn, nbytes):
+    def run(name, fn, nbytes, sample):
         fn()
         reps, t0 = 0, time.perf_counter()
         while True:
@@ -199,33 +501,32 @@ def cpu_extras(budget_s=2.5):
             dt = time.perf_counter() - t0
             if dt > budget_s:
                 break
-        out[name] = {"cpu_GB/s": round(nbytes * reps / dt / 1e9, 2), "cores": 1, "reps": reps}
+        out[name] = {"cpu_GB/s": round(nbytes * reps / dt / 1e9, 2), "cpu_cores": 1, "cpu_sample": "%d x %s" % (reps, sample)}
 
-    # ResNet-50: memcpy pack, ScaleBuffer 0.125 in place, sum with one peer, memcpy unpack (7P)
-    counts = [W.numel(s) for s in W.resnet50_shapes()]
-    ts = [(rng.standard_normal(c, dtype=np.float32) * np.float32(1e-3)) for c in counts]
+    # fusion stress: memcpy pack, ScaleBuffer 0.125 in place, memcpy unpack (4P)
+    counts = W.stress_counts(seed=3)
+    ts = [rng.uniform(-1, 1, c).astype(np.float32) for c in counts]
     outs = [np.empty_like(t) for t in ts]
     n, k = sum(counts), len(counts)
     nb = np.array([4 * c for c in counts], np.int64)
     buf = np.zeros(n, np.float32)
-    peer = rng.standard_normal(n, dtype=np.float32)
     tp, op = ptrs(ts), ptrs(outs)
 
-    def resnet():
+    def stress():
         L.orc_pack(tp, P(nb), c_int(k), P(buf))
         L.orc_scale_buffer(P(buf), P(buf), c_int64(n), c_double(0.125), c_int(F32))
-        L.orc_sum(P(peer), P(buf), c_int64(n), c_int(F32))
         L.orc_unpack(P(buf), op, P(nb), c_int(k))
 
-    run("resnet50_fp32_pack_scale_reduce_unpack", resnet, 7 * 4 * n)
+    run("c2_fusion_stress", stress, 4 * 4 * n, "the whole 1,024-tensor set")
 
     # BERT-large, one cycle of 42 tensors: fp32 -> fp16 with prescale, 7 peers on 1/8, fp16 -> fp32
     counts = [W.numel(s) for s in W.bert_large_shapes()][7:49]
     ts = [(rng.standard_normal(c, dtype=np.float32) * np.float32(1e-4)) for c in counts]
     outs = [np.empty_like(t) for t in ts]
     n = sum(counts)
-    hbuf = np.zeros(n, np.uint16)
-    peers = [rng.integers(0, 0x0400, n // 8, dtype=np.uint16) for _ in range(7)]
+    hbuf = np.zeros(n + 4096, np.uint16)
+    share = W.reduce_scatter_share(n, 8)
+    peers = [rng.integers(0, 0x0400, share, dtype=np.uint16) for _ in range(7)]
 
     def bert():
         off = 0
@@ -233,13 +534,13 @@ def cpu_extras(budget_s=2.5):
             L.orc_scale_cast_f32_to_f16_f16c(P(t), P(hbuf, 2 * off), c_int64(c), c_double(0.125))
             off += c
         for p in peers:
-            L.orc_float16_sum(P(p), P(hbuf), c_int64(n // 8))
+            L.orc_float16_sum(P(p), P(hbuf), c_int64(share))
         off = 0
         for o, c in zip(outs, counts):
             L.orc_scale_cast_f16_to_f32_f16c(P(hbuf, 2 * off), P(o), c_int64(c), c_double(1.0))
             off += c
 
-    run("bert_large_fp32_to_fp16_7peers_eighth_chunk", bert, 6 * n + 9 * 2 * (n // 8) + 6 * n)
+    run("c3_bert_large_fp32_to_fp16_7peers_eighth_share", bert, 6 * n + 9 * 2 * share + 6 * n, "one 42-tensor cycle")
 
     # Adasum: the whole pair, in place on a (values stay finite from repetition to repetition)
     n = 1 << 25
@@ -247,8 +548,9 @@ def cpu_extras(budget_s=2.5):
     a = rng.standard_normal(n, dtype=np.float32)
     b = rng.standard_normal(n, dtype=np.float32)
     nd, co = np.zeros(192), np.zeros(128)
-    run("adasum_fp32_2x32M_64layers",
-        lambda: L.orc_adasum_pairwise(P(a), P(b), c_int(F32), P(lc), c_int(64), P(nd), P(co)), 5 * n * 4)
+    run("c4_adasum_fp32_2x32M_64layers",
+        lambda: L.orc_adasum_pairwise(P(a), P(b), c_int(F32), P(lc), c_int(64), P(nd), P(co)), 5 * n * 4,
+        "the whole pair")
 
     # GPT-2 XL: one transformer layer (12 fp16 tensors, 61.5 MB)
     counts = [W.numel(s) for s in W.gpt2_xl_shapes()][2:14]
@@ -266,17 +568,25 @@ def cpu_extras(budget_s=2.5):
         L.orc_float16_sum(P(peer), P(hbuf), c_int64(n))
         L.orc_unpack(P(hbuf), op2, P(nb), c_int(k))
 
-    run("gpt2_xl_fp16_two_streams", gpt2, 7 * 2 * n)
+    run("c5_gpt2_xl_fp16_two_streams", gpt2, 7 * 2 * n, "one transformer layer (12 tensors)")
     return out
 
 
-def per_tensor_comparator(counts, src, dst, reps=20):
+# ----------------------------------------------------------------------------------------------
+# extras
+# ----------------------------------------------------------------------------------------------
+
+def per_tensor_comparator(reps=20):
     """The fusion stress step through the C++ adapter's GPUAllreduce::Execute twice: with the
     offset-table kernels, and with one hipMemcpyAsync per tensor each way plus a whole-buffer
     ScaleBuffer (HOROVOD_BATCH_D2D_MEMCOPIES=0, what Horovod does on ROCm today,
     ops/gpu_operations.cc:209-222,230-235,327-332).  Both include the op's completion wait."""
     import ctypes
     import torch
+    from horovod_amd import workloads as W
+    counts = W.stress_counts(seed=3)
+    src = DeviceSet(counts, 4, lambda n: randn_bytes(n, torch.float32, 1.0, 4))
+    dst = DeviceSet(counts, 4, zeros_bytes)
     lib = ctypes.CDLL(os.path.join(ROOT, "horovod_amd", "lib", "libhvdhip_adapter.so"))
     lib.hvd_adapter_create.restype = ctypes.c_void_p
     lib.hvd_adapter_create.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p]
@@ -309,129 +619,22 @@ def per_tensor_comparator(counts, src, dst, reps=20):
     return out
 
 
-_PAIR = []
-
-
-def stream_pair():
-    """Two library streams created once, before any other, and shared by everything in this run
-    that alternates over stream slots: streams that are created later, while others exist, can
-    land on a hardware queue that is already in use and then overlap nothing."""
-    if not _PAIR:
-        from horovod_amd import Stream
-        _PAIR.extend([Stream(), Stream()])
-    return _PAIR
-
-
-def extras(steps, warmup):
-    """The other pipelines, each as algorithmic GB/s and fraction of the HBM peak."""
-    import torch
-    from horovod_amd import AdasumPlan, DTYPE, Stream, workloads as W
-    from horovod_amd.pipeline import AllreducePipeline
-    out = {}
-    g = torch.Generator(device="cuda")
-
-    def randn(nbytes, dtype, std, seed):
-        g.manual_seed(seed)
-        n = nbytes // torch.empty(0, dtype=dtype).element_size()
-        return (torch.randn(n, generator=g, device="cuda", dtype=torch.float32) * std).to(dtype).view(torch.uint8)
-
-    def run_pipeline(name, shapes, tdtype, bdtype, std, peers, fraction, streams, kway=True, steps_=steps,
-                     replicas=1):
-        tt = {DTYPE["float32"]: torch.float32, DTYPE["float16"]: torch.float16}
-        es = 4 if tdtype == DTYPE["float32"] else 2
-        counts = [W.numel(s) for s in shapes]
-        reps = []
-        shared = stream_pair()[:streams]  # every replica queues on the same stream(s)
-        for r in range(replicas):
-            src = DeviceSet(counts, es, lambda n: randn(n, tt[tdtype], std, 1 + r))
-            dst = DeviceSet(counts, es, lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
-            pipe = AllreducePipeline(src.ptrs, dst.ptrs, counts, tdtype, bdtype, streams=shared)
-            bs = 4 if pipe.buffer_dtype == DTYPE["float32"] else 2
-            max_elems = max(c.buffer_elems for c in pipe.cycles)
-            peer_bufs = []
-            for p in range(peers):
-                nb = int(max_elems * fraction) * bs + 256
-                peer_bufs.append(randn((nb + 255) // 256 * 256, tt[pipe.buffer_dtype], std, 100 + 16 * r + p))
-            reps.append((src, dst, pipe, peer_bufs))
-        torch.cuda.synchronize()
-        turn = [0]
-
-        def fn():
-            i = turn[0] = (turn[0] + 1) % len(reps)
-            _, _, pipe, peer_bufs = reps[i]
-            pipe.run(0.125, 1.0, (lambda ci, p: peer_bufs[p].data_ptr()) if peers else None, peers, fraction, kway)
-
-        def sync():
-            for _, _, pipe, _ in reps:
-                pipe.synchronize()
-
-        sec = timed(fn, sync, steps_, max(2, warmup // 4))
-        pipe = reps[0][2]
-        ab = pipe.algorithmic_bytes(peers, fraction, kway)
-        out[name] = {"GB/s": round(ab / sec / 1e9, 1), "frac_of_hbm_peak": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4),
-                     "ms": round(sec * 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1), "cycles": len(pipe.cycles),
-                     "streams": streams, "peers": peers, "reduce": "k-way" if kway else "per-peer",
-                     "completion_event_per_cycle": pipe.completion_events,
-                     "replicas_rotated": replicas}
-        for _, _, pipe, _ in reps:
-            pipe.destroy()
-        del reps
-        torch.cuda.empty_cache()
-
-    F32, F16 = DTYPE["float32"], DTYPE["float16"]
-    run_pipeline("resnet50_fp32_pack_scale_reduce_unpack", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0, 1,
-                 replicas=4)
-    run_pipeline("resnet50_fp32_two_streams", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0, 2, replicas=4)
-    run_pipeline("bert_large_fp32_to_fp16_7peers_eighth_chunk", W.bert_large_shapes(), F32, F16, 1e-4, 7, 0.125, 1,
-                 steps_=max(5, steps // 10))
-    run_pipeline("bert_large_fp32_to_fp16_two_streams", W.bert_large_shapes(), F32, F16, 1e-4, 7, 0.125, 2,
-                 steps_=max(5, steps // 10))
-    run_pipeline("gpt2_xl_fp16_two_streams", W.gpt2_xl_shapes(), F16, F16, 1e-3, 1, 1.0, 2,
-                 steps_=max(3, steps // 40))
-
-    # Adasum combine: two fp32 vectors of 2^25 elements, 64 layers, per-layer correlation 0.3;
-    # four independent pairs are rotated so that no pair is still cached when its turn comes again
-    n = 1 << 25
-    counts = W.adasum_layer_counts(n, 64, seed=13)
-    pairs = []
-    for r in range(4):
-        g.manual_seed(14 + 2 * r)
-        a = torch.randn(n, generator=g, device="cuda", dtype=torch.float32)
-        g.manual_seed(15 + 2 * r)
-        b = 0.3 * a + (1 - 0.09) ** 0.5 * torch.randn(n, generator=g, device="cuda", dtype=torch.float32)
-        pairs.append((a, b))
-    plan = AdasumPlan(counts, F32)
-    s = stream_pair()[0]
-    torch.cuda.synchronize()
-    turn = [0]
-
-    def combine():
-        # the combine rewrites a; its cost does not depend on the values, which stay finite
-        i = turn[0] = (turn[0] + 1) % len(pairs)
-        plan.combine(pairs[i][0].data_ptr(), pairs[i][1].data_ptr(), s)
-
-    sec = event_timed(combine, s, max(8, steps // 4), 4)
-    ab = 5 * n * 4
-    out["adasum_fp32_2x32M_64layers"] = {"GB/s": round(ab / sec / 1e9, 1),
-                                         "frac_of_hbm_peak": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4),
-                                         "ms": round(sec * 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1),
-                                         "replicas_rotated": len(pairs)}
-    plan.destroy()
-    del pairs
-    torch.cuda.empty_cache()
-
-    # Allgather fusion buffer (ops/collective_operations.cc:234-288): 8 ranks, 128 entries per rank with
-    # the stress workload's size mix.  This GPU packs its own slab at its displacement (the other
-    # slabs arrive by the collective, which is not built) and unpacks one component per (entry, rank).
-    # Each direction is one batched copy; 4 independent sets are rotated.
+def allgather_extra(steps):
+    """Allgather fusion buffer (ops/collective_operations.cc:234-288): 8 ranks, 128 entries per rank with
+    the stress workload's size mix.  This GPU packs its own slab at its displacement (the other slabs
+    arrive by the collective, which is not built) and unpacks one component per (entry, rank).  Each
+    direction is one batched copy through the descriptor-array entry point; 4 independent sets rotate."""
     import ctypes
+    import torch
     import horovod_amd
+    from horovod_amd import workloads as W
+    s = stream_pair()[0]
     world, es = 8, 4
     counts = W.stress_counts(seed=21, n=128)
     slab = es * sum(counts)
     sets = []
     for r in range(4):
-        src = DeviceSet(counts, es, lambda n: randn(n, torch.float32, 1.0, 60 + r))
+        src = DeviceSet(counts, es, lambda n: randn_bytes(n, torch.float32, 1.0, 60 + r))
         fusion = torch.empty(world * slab, dtype=torch.uint8, device="cuda")
         outs = [torch.empty(world * c * es, dtype=torch.uint8, device="cuda") for c in counts]
         pack_dst, at = [], 3 * slab  # this rank's displacement (rank 3 of 8)
@@ -454,6 +657,7 @@ def extras(steps, warmup):
         sets.append((src, fusion, outs, pack_args, un_args))
     torch.cuda.synchronize()
     copy = horovod_amd.lib().hvdhip_batched_d2d_memcpy
+    turn = [0]
 
     def gather_step():
         i = turn[0] = (turn[0] + 1) % len(sets)
@@ -462,13 +666,83 @@ def extras(steps, warmup):
 
     sec = event_timed(gather_step, s, max(8, steps // 4), 4)
     ab = 2 * slab + 2 * world * slab
-    out["allgather_fusion_8ranks_pack_unpack"] = {
-        "GB/s": round(ab / sec / 1e9, 1), "frac_of_hbm_peak": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4),
-        "ms": round(sec * 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1), "entries": len(counts), "ranks": world,
-        "copies_per_step": len(counts) * (world + 1), "streams": 1, "replicas_rotated": len(sets)}
-    del sets
+    return {"algorithmic_GB/s": round(ab / sec / 1e9, 1),
+            "algorithmic_frac_of_8TBps": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4),
+            "ms": round(sec * 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1), "entries": len(counts), "ranks": world,
+            "copies_per_step": len(counts) * (world + 1), "streams": 1, "replicas_rotated": len(sets)}
+
+
+def extras(headline_cases_block):
+    import torch
+    from horovod_amd import DTYPE, workloads as W
+    F32, F16 = DTYPE["float32"], DTYPE["float16"]
+    out = {}
+
+    def pipeline(name, shapes, tdt, bdt, std, peers, fraction, streams, replicas, steps, arrays=False, note=None):
+        run = PipelineRun(shapes, tdt, bdt, std, peers, fraction, streams, replicas, arrays=arrays)
+        sec = timed(run.one_pass, run.sync, steps, max(2, steps // 10))
+        out[name] = pipeline_figures(run, sec, streams, note)
+        run.destroy()
+
+    def kernels(name, cfg):
+        cases = build_cases(cfg)
+        blocks = measure_cases(cases)
+        release(cases)
+        del cases
+        torch.cuda.empty_cache()
+        out[name]["kernels"] = blocks
+        out[name]["roofline"] = max(blocks, key=lambda b: b["launch_us"])
+        out[name]["traffic_profile"] = TRAFFIC_PROFILE.get(cfg.rstrip("h"))
+
+    # C1 on two streams (the headline is the one-stream figure); its kernel blocks come from the headline
+    pipeline("c1_resnet50_fp32_two_streams", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0, 2, 4, 200)
+    out["c1_resnet50_fp32_two_streams"]["kernels"] = headline_cases_block
+
+    # C2: fusion stress, pack + unpack, 200 repetitions
+    stress = [(c,) for c in W.stress_counts(seed=3)]
+    pipeline("c2_fusion_stress", stress, F32, F32, 1.0, 0, 1.0, 1, 8, 200,
+             note="1,024 fp32 tensors, log-uniform 256..65,536 elements (seed 3): pack with prescale 0.125, unpack; "
+                  "200 repetitions timed; every kernel behind its predecessor on one stream")
+    kernels("c2_fusion_stress", "c2")
+    pipeline("c2_fusion_stress_two_streams", stress, F32, F32, 1.0, 0, 1.0, 2, 8, 200,
+             note="consecutive repetitions alternate over two stream slots, each with its own fusion buffer")
+    try:
+        out["c2_fusion_stress"]["execute_vs_per_tensor_copies"] = per_tensor_comparator()
+    except Exception as e:  # pragma: no cover
+        out["c2_fusion_stress"]["execute_vs_per_tensor_copies"] = {"error": "%s: %s" % (type(e).__name__, e)}
+
+    # C3: BERT-large fp32 -> fp16, 7 peers on the 1/8 share
+    pipeline("c3_bert_large_fp32_to_fp16_7peers_eighth_share", W.bert_large_shapes(), F32, F16, 1e-4, 7, 0.125, 1, 1, 20)
+    kernels("c3_bert_large_fp32_to_fp16_7peers_eighth_share", "c3")
+    pipeline("c3_bert_large_two_streams", W.bert_large_shapes(), F32, F16, 1e-4, 7, 0.125, 2, 1, 20)
+
+    # C4: Adasum combine, fp32 (the configuration) and fp16
+    for cfg, name in (("c4", "c4_adasum_fp32_2x32M_64layers"), ("c4h", "c4_adasum_fp16_2x32M_64layers")):
+        cases = build_cases(cfg)
+        blocks = measure_cases(cases, steps=50, warmup=4)
+        release(cases)
+        del cases
+        torch.cuda.empty_cache()
+        b = blocks[0]
+        out[name] = {"algorithmic_GB/s": b["achieved"], "algorithmic_frac_of_8TBps": b["frac"],
+                     "ms": round(b["launch_us"] / 1e3, 4), "algorithmic_MB": round(b["algorithmic_bytes_per_launch"] / 1e6, 1),
+                     "replicas_rotated": 4, "kernels": blocks, "roofline": b, "traffic_profile": TRAFFIC_PROFILE["c4"],
+                     "note": "two launches timed together with HIP events; per-kernel durations and traffic are in the profile"}
+
+    # C5: GPT-2 XL fp16 on two streams (the configuration), on one, and through the array-taking entry points
+    pipeline("c5_gpt2_xl_fp16_two_streams", W.gpt2_xl_shapes(), F16, F16, 1e-3, 1, 1.0, 2, 1, 5)
+    kernels("c5_gpt2_xl_fp16_two_streams", "c5")
+    pipeline("c5_gpt2_xl_fp16_one_stream", W.gpt2_xl_shapes(), F16, F16, 1e-3, 1, 1.0, 1, 1, 5)
+    pipeline("c5_gpt2_xl_fp16_array_entry_points", W.gpt2_xl_shapes(), F16, F16, 1e-3, 1, 1.0, 2, 1, 5, arrays=True,
+             note="pack and unpack of every cycle through hvdhip_batched_scaled_d2d_memcpy (the by-value launchers "
+                  "of ops/gpu_operations.cc:186-206) instead of explicit plans: 96 distinct copy sets per step, "
+                  "their tables resident in the library's cache after the first step")
+
+    out["allgather_fusion_8ranks_pack_unpack"] = allgather_extra(200)
     return out
 
+
+# ----------------------------------------------------------------------------------------------
 
 def main():
     args = parse()
@@ -481,7 +755,7 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     import horovod_amd
-    from horovod_amd import DTYPE, FusionPlan, Stream
+    from horovod_amd import DTYPE, workloads as W
     from horovod_amd import build as native
     native.ensure_built()  # loads what is built; builds only if nothing is
     horovod_amd.lib()  # fails loudly if the HIP library cannot be loaded
@@ -499,137 +773,71 @@ def main():
         stream.synchronize()
         return
 
-    if args.kernel_only in ("reduce", "adasum"):
-        from horovod_amd import AdasumPlan, host as H, workloads as W
-        g = torch.Generator(device="cuda")
-        g.manual_seed(7)
-        n = (64 << 20) // 4 if args.kernel_only == "reduce" else 1 << 25
-        pairs = [(torch.randn(n, generator=g, device="cuda"), torch.randn(n, generator=g, device="cuda"))
-                 for _ in range(4)]
-        plan = AdasumPlan(W.adasum_layer_counts(n, 64, seed=13), F32) if args.kernel_only == "adasum" else None
-        torch.cuda.synchronize()
-        for i in range(args.warmup + args.steps):
-            a, b = pairs[i % 4]
-            if plan is None:
-                H.reduce_sum(a.data_ptr(), b.data_ptr(), n, F32, stream)
-            else:
-                plan.combine(a.data_ptr(), b.data_ptr(), stream)
-        stream.synchronize()
+    if args.kernel_only:
+        for c in build_cases(args.kernel_only):
+            for _ in range(args.warmup + args.steps):
+                c.fn()
+            stream.synchronize()
         return
 
-    counts, host, sets = stress_workload(max(1, args.replicas))
-    plans = [FusionPlan(src.ptrs, dst.ptrs, counts, F32) for src, dst in sets]
-    # One fusion buffer per stream slot, reused by every repetition: Horovod's FusionBufferManager keeps
-    # one per (device, framework, stream slot) for the life of the job (ops/gpu_operations.cc:122-124).
-    # The gradient tensors on either side of it rotate over the replicas.
-    fbs = [torch.empty(plans[0].buffer_len, dtype=torch.uint8, device="cuda") for _ in range(2)]
-    plan = plans[0]
-    payload = 4 * sum(counts)
-    torch.cuda.synchronize()
-    turn = [0]
-
-    def pack():
-        i = turn[0] = (turn[0] + 1) % len(plans)
-        plans[i].pack(fbs[0].data_ptr(), 0.125, stream)
-
-    if args.streams not in (1, 2):
-        print("bench.py alternates over one or two stream slots", file=sys.stderr)
-        sys.exit(2)
-    slots = stream_pair()[:args.streams]
+    # ---- headline: C1, the whole pipeline on one stream
+    run = PipelineRun(W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0, 1, 4)
 
     def step():
         for _ in range(REPS):
-            i = turn[0] = (turn[0] + 1) % len(plans)
-            plans[i].pack(fbs[i % len(slots)].data_ptr(), 0.125, slots[i % len(slots)])
-            plans[i].unpack(fbs[i % len(slots)].data_ptr(), 1.0, slots[i % len(slots)])
+            run.one_pass()
 
-    def sync_slots():
-        for st in slots:
-            st.synchronize()
+    sec = timed(step, run.sync, args.steps, args.warmup)
+    ab = run.algorithmic_bytes()
+    value = REPS * ab / sec / 1e9
+    payload = 4 * sum(run.counts)
+    config = {"workload": "C1: ResNet-50 fp32 gradients, 161 tensors, 25,557,032 elements, N(0,1e-3); fused by the "
+                          "reference's planner at a 64 MiB threshold into %d cycles; per cycle pack with prescale 0.125 "
+                          "-> reduce-sum of the whole buffer with one peer buffer resident on the device -> unpack "
+                          "(postscale 1.0); all on one stream, the stream slot's one persistent fusion buffer; the "
+                          "tensor sets (inputs, outputs, peers) rotate over %d replicas so that no pass finds its "
+                          "inputs in the 256 MB Infinity Cache" % (len(run.pipe.cycles), len(run.reps)),
+              "tensors": len(run.counts), "payload_bytes": payload, "cycles": len(run.pipe.cycles),
+              "cycle_buffer_bytes": [c.plan.buffer_len for c in run.pipe.cycles], "fusion_threshold": W.FUSION_THRESHOLD,
+              "peers": 1, "prescale": 0.125, "postscale": 1.0, "passes_per_step": REPS,
+              "algorithmic_bytes_per_pass": ab, "algorithmic_bytes_per_step": REPS * ab, "replicas_rotated": len(run.reps),
+              "streams": 1,
+              "value_is": "algorithmic bytes (pack P_in+P_buf, reduce 3C, unpack P_buf+P_out = 7P) / wall time; within a "
+                          "cycle the fusion buffer passes from kernel to kernel through the Infinity Cache, so this is "
+                          "not an HBM counter; the HBM claim is roofline.frac"}
+    run.destroy()
 
-    if args.kernel_only:
-        for _ in range(args.warmup + args.steps):
-            pack()
-        stream.synchronize()
-        return
-
-    sec = timed(step, sync_slots, args.steps, args.warmup)
-    value = REPS * 4 * payload / sec / 1e9
-
-    ksec = event_timed(pack, stream, 200, 20)
-    achieved = 2 * payload / ksec / 1e9
-    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": PACK_TRAFFIC_BYTES_MEASURED,
-                "kernel": "xfer_k<Scale<float,float>, pack, write-through stores>", "launch_us": round(ksec * 1e6, 2),
-                "timed": "launched back to back on one stream: tensors of another replica every launch, "
-                         "the stream slot's one fusion buffer as the destination",
-                "algorithmic_bytes_per_launch": 2 * payload, "workgroups": plan.num_chunks}
+    # ---- roofline: every kernel of the C1 cycle, the dominant one as the headline's block
+    cases = build_cases("c1")
+    blocks = measure_cases(cases, steps=200, warmup=20)
+    release(cases)
+    del cases
+    torch.cuda.empty_cache()
+    roofline = dict(next(b for b in blocks if b["case"] == "c1.reduce"))
+    roofline["why_this_kernel"] = ("the reduce-sum takes the largest share of the pipeline's kernel time (3C of the "
+                                   "7P algorithmic bytes)")
 
     result = {
         "metric": "achieved HBM GB/s (% of 8 TB/s) for fused pack+scale+reduce+unpack; Adasum GB/s",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(sec * 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "fusion stress: 1,024 fp32 tensors, log-uniform 256..65,536 elements (seed 3), "
-                               "U(-1,1) (seed 4); pack with prescale 0.125 into the fusion buffer, unpack, 200 repetitions; "
-                               "consecutive repetitions alternate over the stream slots, each slot with its own persistent "
-                               "fusion buffer (as FusionBufferManager keeps them); the tensors rotate over the replicas",
-                   "tensors": len(counts), "payload_bytes": payload, "buffer_len": plan.buffer_len,
-                   "repetitions_per_step": REPS, "algorithmic_bytes_per_step": REPS * 4 * payload,
-                   "replicas_rotated": len(plans),
-                   "streams": len(slots)},
-        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "dtype": "f32", "data": "synthetic", "config": config,
+        "algorithmic_frac_of_8TBps": round(value / HBM_PEAK_GBS, 4),
         "roofline": roofline,
+        "traffic_profile": TRAFFIC_PROFILE["c1"],
     }
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline_stress(counts, host)
-    other = None
+        result["cpu_baseline"] = cpu_baseline_resnet()
     if not args.no_extra:
-        # The same steps with the other stream count: all on one stream when the headline alternates over
-        # several (every kernel then waits for its predecessor, the reference's default
-        # HOROVOD_NUM_NCCL_STREAMS=1), or on two streams when the headline was asked to use one.
+        # the extra configurations must never cost the headline line
         try:
-            alt = stream_pair()[:1 if len(slots) > 1 else 2]
-
-            def step_alt():
-                for _ in range(REPS):
-                    i = turn[0] = (turn[0] + 1) % len(plans)
-                    plans[i].pack(fbs[i % len(alt)].data_ptr(), 0.125, alt[i % len(alt)])
-                    plans[i].unpack(fbs[i % len(alt)].data_ptr(), 1.0, alt[i % len(alt)])
-
-            def sync_alt():
-                for st in alt:
-                    st.synchronize()
-
-            sec2 = timed(step_alt, sync_alt, args.steps, args.warmup)
-            other = {"GB/s": round(REPS * 4 * payload / sec2 / 1e9, 1),
-                     "frac_of_hbm_peak": round(REPS * 4 * payload / sec2 / 1e9 / HBM_PEAK_GBS, 4),
-                     "ms_per_step": round(sec2 * 1e3, 5), "streams": len(alt)}
-        except Exception as e:  # pragma: no cover
-            other = {"error": "%s: %s" % (type(e).__name__, e)}
-    comparator = None
-    if not args.no_extra:
-        try:
-            comparator = per_tensor_comparator(counts, sets[0][0], sets[0][1])
-        except Exception as e:  # pragma: no cover
-            comparator = {"error": "%s: %s" % (type(e).__name__, e)}
-    for p in plans:
-        p.destroy()
-    del fbs, sets
-    torch.cuda.empty_cache()
-    if not args.no_extra:
-        # the extra pipelines must never cost the headline line
-        try:
-            result["extra"] = extras(200, 20)
+            result["extra"] = extras(blocks)
         except Exception as e:  # pragma: no cover
             result["extra"] = {"error": "%s: %s" % (type(e).__name__, e)}
-        result["extra"]["fusion_stress_execute_vs_per_tensor_copies"] = comparator
-        result["extra"]["fusion_stress_one_stream" if len(slots) > 1 else "fusion_stress_two_streams"] = other
         if not args.no_cpu and "error" not in result["extra"]:
             try:
                 for name, v in cpu_extras().items():
-                    result["extra"][name].update({"cpu_GB/s": v["cpu_GB/s"], "cpu_cores": 1,
-                                                  "cpu_sample_reps": v["reps"]})
+                    result["extra"][name].update(v)
             except Exception as e:  # pragma: no cover
                 result["extra"]["cpu_error"] = "%s: %s" % (type(e).__name__, e)
     print(json.dumps(result))

@@ -205,7 +205,7 @@ struct Axpby<half_t> {
 // data loads are in flight, which saves the finalize launch between the two passes.  All
 // workgroups of a layer execute the same additions in the same order, so they agree to the
 // bit; the layer's first workgroup also stores the sums and coefficients for readers.
-template <typename T, bool FUSED, bool WT>
+template <typename T, bool FUSED, int ST>
 __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ chunks, T* a,
                                                     const T* __restrict__ b,
                                                     const double* __restrict__ coeffs,
@@ -222,7 +222,7 @@ __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ ch
   gptr<T> pa = as_global(a + c.tensor);
   gptr<const T> pb = as_global(b + c.tensor);
   const uint32_t nv = n / VEC;
-  const Window out = store_window<WT>(pa, n * (uint32_t)sizeof(T));
+  const Window out = store_window<ST>(pa, n * (uint32_t)sizeof(T));
   uint32_t v = threadIdx.x;
   double ca, cb;
   if (FUSED) {
@@ -284,7 +284,7 @@ __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ ch
       for (int u = 0; u < kUnroll; ++u) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) x[u].v[j] = Axpby<T>::f(ca, x[u].v[j], cb, y[u].v[j]);
-        stw<WT, T, VEC>(out, (v + u * kWG) * 16u, x[u]);
+        stw<ST, T, VEC>(out, (v + u * kWG) * 16u, x[u]);
       }
       v += kUnroll * kWG;
     }
@@ -304,7 +304,7 @@ __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ ch
     for (int u = 0; u < kUnroll; ++u) {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) x[u].v[j] = Axpby<T>::f(ca, x[u].v[j], cb, y[u].v[j]);
-      stw<WT, T, VEC>(out, (v + u * kWG) * 16u, x[u]);
+      stw<ST, T, VEC>(out, (v + u * kWG) * 16u, x[u]);
     }
   }
   for (; v < nv; v += kWG) {
@@ -312,7 +312,7 @@ __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ ch
     const V y = ldv<T, VEC>(pb + (size_t)v * VEC);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) x.v[j] = Axpby<T>::f(ca, x.v[j], cb, y.v[j]);
-    stw<WT, T, VEC>(out, v * 16u, x);
+    stw<ST, T, VEC>(out, v * 16u, x);
   }
   const uint32_t t = nv * VEC + threadIdx.x;
   if (t < n) pa[t] = Axpby<T>::f(ca, pa[t], cb, pb[t]);
@@ -414,14 +414,11 @@ template <typename T, bool FUSED>
 void launch_scaled_add(hvdhip_adasum_plan* p, void* a, const void* b, const double* coeffs,
                        double ca, double cb, hipStream_t s) {
   const DevTables& t = p->tables;
-  if (write_through(Stores::kAdasum))
-    launch(scaled_add_k<T, FUSED, true>, t.nchunks, s, t.chunks,
-                       static_cast<T*>(a), static_cast<const T*>(b), coeffs, ca, cb, p->layers,
-                       p->partials, p->normdots, p->coeffs, std::sqrt(DBL_MIN), (uint32_t)p->nlayers);
-  else
-    launch(scaled_add_k<T, FUSED, false>, t.nchunks, s, t.chunks,
-                       static_cast<T*>(a), static_cast<const T*>(b), coeffs, ca, cb, p->layers,
-                       p->partials, p->normdots, p->coeffs, std::sqrt(DBL_MIN), (uint32_t)p->nlayers);
+  with_store_policy(Stores::kAdasum, [&](auto st) {
+    launch(scaled_add_k<T, FUSED, decltype(st)::value>, t.nchunks, s, t.chunks, static_cast<T*>(a),
+           static_cast<const T*>(b), coeffs, ca, cb, p->layers, p->partials, p->normdots, p->coeffs,
+           std::sqrt(DBL_MIN), (uint32_t)p->nlayers);
+  });
 }
 
 template <bool FUSED>

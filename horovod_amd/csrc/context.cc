@@ -125,22 +125,24 @@ uint32_t xcd_run(uint64_t nchunks, uint32_t chunk_bytes, bool long_runs) {
   return bytes > chunk_bytes ? bytes / chunk_bytes : 1;
 }
 
-bool write_through(Stores family) {
-  constexpr unsigned kDefaultMask = 1u << (unsigned)Stores::kPack | 1u << (unsigned)Stores::kPackNarrowing |
-                                    1u << (unsigned)Stores::kReduceFew | 1u << (unsigned)Stores::kReduceMany;
-  static const unsigned mask = [] {
+int store_policy(Stores family) {
+  constexpr unsigned kDefaultThrough = 1u << (unsigned)Stores::kPack | 1u << (unsigned)Stores::kPackNarrowing |
+                                       1u << (unsigned)Stores::kReduceFew | 1u << (unsigned)Stores::kReduceMany;
+  static const unsigned through = [] {
     const char* e = std::getenv("HVDHIP_WRITE_THROUGH");
-    return e ? (unsigned)std::strtoul(e, nullptr, 0) : kDefaultMask;
+    return e ? (unsigned)std::strtoul(e, nullptr, 0) : kDefaultThrough;
   }();
-  return (mask >> (unsigned)family) & 1u;
+  return (through >> (unsigned)family) & 1u;
 }
 
-uint32_t xcd_shift(uint64_t nblocks, uint32_t tile_bytes) {
+XcdOrder xcd_order(uint64_t nblocks, uint32_t tile_bytes) {
   const uint32_t run = xcd_run(nblocks, tile_bytes);
-  if (run == 0 || (run & (run - 1)) != 0) return kNoXcdOrder;
-  uint32_t shift = 0;
-  while ((1u << shift) < run) ++shift;
-  return shift;
+  XcdOrder o = {0, 0};
+  if (run == 0 || (run & (run - 1)) != 0) return o;  // natural order
+  while ((1u << o.shift) < run) ++o.shift;
+  const uint64_t group = (uint64_t)kXcds << o.shift;
+  o.ordered = (uint32_t)(nblocks / group * group);
+  return o;
 }
 
 void fill_chunks(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t tensor_es,

@@ -7,6 +7,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "hvdhip.h"
@@ -111,16 +112,19 @@ __host__ __device__ inline uint64_t xcd_slot(uint64_t chunk, uint64_t nchunks, u
   return chunk - w + (w % run) * kXcds + w / run;
 }
 
-// The same mapping for kernels that number their tiles themselves, in shifts and masks: shift =
-// log2(run) for a power-of-two run, kNoXcdOrder for workgroup order = tile order.
-constexpr uint32_t kNoXcdOrder = 32;
-uint32_t xcd_shift(uint64_t nblocks, uint32_t tile_bytes);
-__device__ inline uint32_t xcd_tile(uint32_t block, uint32_t nblocks, uint32_t shift) {
-  if (shift >= kNoXcdOrder) return block;
-  const uint32_t mask = (kXcds << shift) - 1;  // group of 8 * run tiles
-  if (block >= (nblocks & ~mask)) return block;
+// The same mapping for kernels that number their tiles themselves, in shifts and masks and without a
+// branch (nothing may stand between a workgroup's start and its first loads): the first `ordered`
+// workgroups (a multiple of 8 << shift, 0 for natural order) are permuted in groups of 8 << shift.
+struct XcdOrder {
+  uint32_t shift;    // log2 of the run length in tiles
+  uint32_t ordered;  // workgroups below this number are permuted
+};
+XcdOrder xcd_order(uint64_t nblocks, uint32_t tile_bytes);
+__device__ __forceinline__ uint32_t xcd_tile(uint32_t block, XcdOrder o) {
+  const uint32_t mask = (kXcds << o.shift) - 1;  // group of 8 * run tiles
   const uint32_t w = block & mask;
-  return block - w + ((w & (kXcds - 1)) << shift) + (w >> 3);
+  const uint32_t permuted = block - w + ((w & (kXcds - 1)) << o.shift) + (w >> 3);
+  return block < o.ordered ? permuted : block;
 }
 
 // Launches a streaming kernel: workgroups of kWG lanes, no dynamic LDS.
@@ -129,19 +133,14 @@ inline void launch(void (*kernel)(KArgs...), uint32_t workgroups, hipStream_t st
   hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(kWG), 0, stream, KArgs(args)...);
 }
 
-// Store policy per kernel family: true = write-through buffer stores, false = non-temporal
-// global stores (vecmem.h).  Lines written through are installed in the 256 MB Infinity Cache on
-// their way to HBM, so a kernel that runs next on the same stream and reads them (the collective
-// or reduce-sum after a pack, the unpack after a reduce-sum) finds them there; non-temporal stores
-// bypass it.  Installing costs the writer something (a stress-workload pack launched back to back
-// with nothing reading its output: 18.0 instead of 16.3 us) and saves the reader more (the unpack
-// behind it: 12 instead of 16.4 us), so the kernels whose output the next kernel reads write
-// through, and the ones whose output leaves the pipeline (unpack, batched copies, Adasum's scaled
-// add, a whole-buffer scale) do not.  Measured per family on the pipelines of bench.py, each bit on
-// its own against all off: pack +3 % (two stream slots) to +9 % (one) on the stress workload,
-// +5-7 % on ResNet-50 and GPT-2 XL; narrowing pack +5-8 % on BERT-large; reduce-sum of one peer
-// +6-7 % on ResNet-50 and GPT-2 XL, of seven peers +1 %; unpack 0 to -2 %, widening unpack -4 to
-// -7 %, batched copies -16 %, scaled add -14 %, whole-buffer scale +-0.
+// Store policy per kernel family (the three kinds of store are described in vecmem.h).  Lines
+// written through are installed in the 256 MB Infinity Cache on their way to HBM, so a kernel that
+// runs next on the same stream and reads them (the collective or reduce-sum after a pack, the unpack
+// after a reduce-sum) finds them there; non-temporal stores bypass it.  Installing costs the writer
+// something (a stress-workload pack launched back to back with nothing reading its output: 18.0
+// instead of 16.3 us) and saves the reader more (the unpack behind it: 12 instead of 16.4 us), so the
+// kernels whose output the next kernel reads write through, and the ones whose output leaves the
+// pipeline (unpack, batched copies, Adasum's scaled add, a whole-buffer scale) do not.
 // HVDHIP_WRITE_THROUGH=<mask> (bit = enumerator value) overrides the built-in table, for tuning.
 enum class Stores {
   kPack = 0,        // same-width pack into the fusion buffer
@@ -154,7 +153,16 @@ enum class Stores {
   kReduceMany = 7,  // reduce-sum of three to eight peers
   kAdasum = 8,      // scaled add
 };
-bool write_through(Stores family);
+int store_policy(Stores family);  // a StorePolicy value
+
+// Calls f(std::integral_constant<int, policy>) for the family's policy.
+template <typename F>
+inline void with_store_policy(Stores family, F&& f) {
+  if (store_policy(family))
+    f(std::integral_constant<int, 1>());
+  else
+    f(std::integral_constant<int, 0>());
+}
 
 // One contiguous run of elements to transfer (host side only).  `tensor` and
 // `output` are absolute device addresses; `off` is a byte offset into the

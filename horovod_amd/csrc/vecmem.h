@@ -116,12 +116,19 @@ __device__ __forceinline__ Arr<T, N> ldw(const ReadWindow& w, uint32_t off) {
   return __builtin_bit_cast(Arr<T, N>, __builtin_amdgcn_raw_buffer_load_b128(w.rsrc, (int)off, 0, kNonTemporal));
 }
 
-// A window over a workgroup's destination range, for stores with a choice of cache policy.
-// WT = false: non-temporal global stores (the lines stay in L2 until they are written back).
-// WT = true: raw buffer stores with the sc0 and sc1 bits, which write the lines through.  Which
-// of the two streams faster depends on the kernel and on what runs around it (measured per
-// kernel family; the table is in context.cc).  A buffer instruction takes its cache policy as an
-// immediate, which is why the write-through path uses one; the window's base must be uniform
+// How a streaming kernel stores.
+//   kStoreNT: non-temporal global stores (the lines bypass the Infinity Cache on their way out).
+//   kStoreWT: raw buffer stores with the sc0 and sc1 bits, which write the lines through L2 at once
+//             and install them in the Infinity Cache, where the next kernel finds them.
+// Which one streams faster depends on the kernel and on what runs around it (measured per kernel
+// family; the table is in context.cc).  Plain stores, which leave the lines in L2 until they are
+// written back, are slower than either once the data is not all zeros (a 62 MB reduce-sum: 29.8 us
+// against 29.3 and 29.8; with zeros everywhere they measure 27.0 us, which is worth knowing before
+// trusting a microbenchmark on freshly cleared memory) and cost a pipeline 4-7 %.
+enum StorePolicy : int { kStoreNT = 0, kStoreWT = 1 };
+
+// A window over a workgroup's destination range.  A buffer instruction takes its cache policy as
+// an immediate, which is why the write-through path uses one; the window's base must be uniform
 // over the wavefront (the resource lives in scalar registers), and stores beyond `bytes` are
 // dropped by the hardware's range check.
 struct Window {
@@ -129,11 +136,11 @@ struct Window {
   uint64_t base;
 };
 
-template <bool WT, typename T>
+template <int ST, typename T>
 __device__ __forceinline__ Window store_window(gptr<T> base, uint32_t bytes) {
   Window w;
   w.base = reinterpret_cast<uint64_t>(base);
-  if constexpr (WT) {
+  if constexpr (ST == kStoreWT) {
     // word 3: 32-bit data format, raw (unstrided, untyped) addressing
     w.rsrc = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(w.base), 0, (int)bytes, 0x00020000);
   }
@@ -141,14 +148,14 @@ __device__ __forceinline__ Window store_window(gptr<T> base, uint32_t bytes) {
 }
 
 // Stores N elements of T at byte offset `off` of the window.
-template <bool WT, typename T, int N>
+template <int ST, typename T, int N>
 __device__ __forceinline__ void stw(const Window& w, uint32_t off, const Arr<T, N>& a) {
-  if constexpr (WT) {
+  if constexpr (ST == kStoreWT) {
+    typedef typename RawSel<(int)sizeof(T) * N>::type R;
 #ifndef HVDHIP_WT_AUX
 #define HVDHIP_WT_AUX (1 | 16)  // sc0 | sc1
 #endif
     constexpr int kScopeBits = HVDHIP_WT_AUX;
-    typedef typename RawSel<(int)sizeof(T) * N>::type R;
     const R r = __builtin_bit_cast(R, a);
     if constexpr (sizeof(T) * N == 16) {
       __builtin_amdgcn_raw_buffer_store_b128(r, w.rsrc, (int)off, 0, kScopeBits);

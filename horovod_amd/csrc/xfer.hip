@@ -134,7 +134,7 @@ struct UnpackF16F32 {
 constexpr int kUnroll = HVDHIP_XFER_UNROLL;  // 16-byte loads in flight per lane
 
 // Streams n elements from src to dst through Op::f with the whole workgroup.
-template <class Op, bool WT>
+template <class Op, int ST>
 __device__ __forceinline__ void stream_range(gptr<const typename Op::S> src,
                                              gptr<typename Op::D> dst, uint32_t n,
                                              typename Op::P p) {
@@ -145,7 +145,7 @@ __device__ __forceinline__ void stream_range(gptr<const typename Op::S> src,
   // of an iteration's vectors before it stores any, and touches no address
   // another lane touches.
   const uint32_t nv = n / VEC;
-  const Window out = store_window<WT>(dst, n * (uint32_t)sizeof(D));
+  const Window out = store_window<ST>(dst, n * (uint32_t)sizeof(D));
   constexpr bool kBytes = sizeof(S) == 1;  // byte elements are read through a window (vecmem.h)
   ReadWindow in;
   if constexpr (kBytes) in = load_window(src, n);
@@ -166,7 +166,7 @@ __device__ __forceinline__ void stream_range(gptr<const typename Op::S> src,
       Arr<D, VEC> y;
 #pragma unroll
       for (int j = 0; j < VEC; ++j) y.v[j] = Op::f(x[u].v[j], p);
-      stw<WT, D, VEC>(out, (v + u * kWG) * (uint32_t)(VEC * sizeof(D)), y);
+      stw<ST, D, VEC>(out, (v + u * kWG) * (uint32_t)(VEC * sizeof(D)), y);
     }
   }
   for (; v < nv; v += kWG) {
@@ -174,7 +174,7 @@ __device__ __forceinline__ void stream_range(gptr<const typename Op::S> src,
     Arr<D, VEC> y;
 #pragma unroll
     for (int j = 0; j < VEC; ++j) y.v[j] = Op::f(x.v[j], p);
-    stw<WT, D, VEC>(out, v * (uint32_t)(VEC * sizeof(D)), y);
+    stw<ST, D, VEC>(out, v * (uint32_t)(VEC * sizeof(D)), y);
   }
   const uint32_t t = nv * VEC + threadIdx.x;  // fewer than VEC elements remain
   if (t < n) dst[t] = Op::f(src[t], p);
@@ -186,7 +186,7 @@ enum Mode { kPack = 0, kUnpack = 1, kDirect = 2 };
 //   kPack:   src = chunk.tensor,      dst = base + chunk.off (pad bytes zeroed)
 //   kUnpack: src = base + chunk.off,  dst = chunk.output
 //   kDirect: src = chunk.tensor,      dst = chunk.output
-template <class Op, int MODE, bool WT>
+template <class Op, int MODE, int ST>
 __global__ __launch_bounds__(kWG) void xfer_k(const Chunk* __restrict__ chunks, uint64_t base,
                                               typename Op::P p) {
   typedef typename Op::S S;
@@ -194,20 +194,20 @@ __global__ __launch_bounds__(kWG) void xfer_k(const Chunk* __restrict__ chunks, 
   const Chunk c = chunks[blockIdx.x];
   const uint64_t src_addr = (MODE == kUnpack) ? base + c.off : c.tensor;
   const uint64_t dst_addr = (MODE == kPack) ? base + c.off : c.output;
-  stream_range<Op, WT>(as_global<const S>(src_addr), as_global<D>(dst_addr), c.n, p);
+  stream_range<Op, ST>(as_global<const S>(src_addr), as_global<D>(dst_addr), c.n, p);
   if (MODE == kPack && threadIdx.x < c.pad)
     as_global<uint8_t>(dst_addr)[(uint64_t)c.n * sizeof(D) + threadIdx.x] = 0;
 }
 
 // Contiguous buffer: workgroup b handles tile t = xcd_tile(b), elements [t*tile, (t+1)*tile).
-template <class Op, bool WT>
-__global__ __launch_bounds__(kWG) void contig_k(const typename Op::S* src,
-                                                typename Op::D* dst, uint64_t n,
-                                                uint32_t tile, uint32_t run, typename Op::P p) {
-  const uint64_t start = (uint64_t)xcd_tile(blockIdx.x, gridDim.x, run) * tile;
+template <class Op, int ST>
+__global__ __launch_bounds__(kWG) void contig_k(const typename Op::S* src, typename Op::D* dst, uint64_t n,
+                                                uint32_t tile, uint32_t shift, uint32_t ordered,
+                                                typename Op::P p) {
+  const uint64_t start = (uint64_t)xcd_tile(blockIdx.x, XcdOrder{shift, ordered}) * tile;
   const uint64_t left = n - start;
   const uint32_t m = left < tile ? (uint32_t)left : tile;
-  stream_range<Op, WT>(as_global(src + start), as_global(dst + start), m, p);
+  stream_range<Op, ST>(as_global(src + start), as_global(dst + start), m, p);
 }
 
 // ----------------------------------------------------------------------
@@ -221,10 +221,9 @@ int launch_xfer(const DevTables& t, uint64_t base, typename Op::P p, hipStream_t
   const Stores family = MODE == kDirect ? Stores::kDirect
                         : MODE == kPack ? (converting ? Stores::kPackNarrowing : Stores::kPack)
                                         : (converting ? Stores::kUnpackWidening : Stores::kUnpack);
-  if (write_through(family))
-    launch(xfer_k<Op, MODE, true>, t.nchunks, stream, t.chunks, base, p);
-  else
-    launch(xfer_k<Op, MODE, false>, t.nchunks, stream, t.chunks, base, p);
+  with_store_policy(family, [&](auto st) {
+    launch(xfer_k<Op, MODE, decltype(st)::value>, t.nchunks, stream, t.chunks, base, p);
+  });
   HVDHIP_CHECK_LAUNCH("xfer_k");
   return 0;
 }
@@ -275,10 +274,10 @@ int launch_contig(const void* in, void* out, int64_t n, typename Op::P p, hipStr
   while (left > 0) {  // one launch unless the buffer needs more than kMaxWorkgroups workgroups
     const uint64_t slice = std::min<uint64_t>(left, kMaxWorkgroups * tile);
     const uint32_t blocks = (uint32_t)((slice + tile - 1) / tile);
-    if (write_through(Stores::kContig))
-      launch(contig_k<Op, true>, blocks, stream, src, dst, slice, tile, xcd_shift(blocks, chunk_bytes(Family::kXfer)), p);
-    else
-      launch(contig_k<Op, false>, blocks, stream, src, dst, slice, tile, xcd_shift(blocks, chunk_bytes(Family::kXfer)), p);
+    const XcdOrder order = xcd_order(blocks, chunk_bytes(Family::kXfer));
+    with_store_policy(Stores::kContig, [&](auto st) {
+      launch(contig_k<Op, decltype(st)::value>, blocks, stream, src, dst, slice, tile, order.shift, order.ordered, p);
+    });
     HVDHIP_CHECK_LAUNCH("contig_k");
     src += slice;
     dst += slice;

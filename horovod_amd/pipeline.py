@@ -43,14 +43,23 @@ class AllreducePipeline:
     share)."""
 
     def __init__(self, tensor_ptrs, output_ptrs, counts, tensor_dtype, buffer_dtype=None,
-                 threshold=FUSION_THRESHOLD, num_streams=1, completion_events=None, streams=None):
+                 threshold=FUSION_THRESHOLD, num_streams=1, completion_events=None, streams=None,
+                 buffers=None, array_entry_points=False):
         """completion_events: record a pooled event after every cycle and wait on those in
         synchronize(), as GPUOpContext::FinalizeGPUQueue does (about 2 us of stream time per
         event).  Default: on when cycles alternate over several streams, off for one stream,
         where synchronize() simply waits for the stream.
 
         streams: existing Stream objects to run on instead of creating num_streams new ones
-        (they stay with the caller), so that several pipelines queue on the same streams."""
+        (they stay with the caller), so that several pipelines queue on the same streams.
+
+        buffers: the fusion buffers of another pipeline on the same streams, one per stream slot, to
+        share instead of allocating new ones (the reference keeps one fusion buffer per stream slot
+        for every response that runs there, ops/gpu_operations.cc:122-124).
+
+        array_entry_points: pack and unpack through hvdhip_batched_scaled_d2d_memcpy, the launcher
+        that takes the copies as arrays with every call (ops/gpu_operations.cc:186-206), instead of
+        explicit plans; same-dtype buffers only."""
         self.tensor_dtype = int(tensor_dtype)
         self.buffer_dtype = int(tensor_dtype if buffer_dtype is None else buffer_dtype)
         ts, bs = dtype_size(self.tensor_dtype), dtype_size(self.buffer_dtype)
@@ -78,8 +87,30 @@ class AllreducePipeline:
         self.completion_events = (num_streams > 1) if completion_events is None else bool(completion_events)
         self.pending = []  # (stream, event) recorded after each cycle
         # room for the dummy elements a reduce-scatter over up to 64 ranks may append (64 * 64 elements)
-        self.buffers = [torch.zeros(max(max_len, 16) + 4096 * bs, dtype=torch.uint8, device="cuda")
-                        for _ in range(num_streams)]
+        need = max(max_len, 16) + 4096 * bs
+        if buffers is not None:
+            if len(buffers) != num_streams or any(b.numel() < need for b in buffers):
+                raise ValueError("shared fusion buffers must be one per stream slot and large enough")
+            self.buffers = list(buffers)
+        else:
+            self.buffers = [torch.zeros(need, dtype=torch.uint8, device="cuda") for _ in range(num_streams)]
+        self.array_entry_points = bool(array_entry_points)
+        if self.array_entry_points:
+            if self.buffer_dtype != self.tensor_dtype:
+                raise ValueError("the array-taking copies do not convert between dtypes")
+            # the descriptor arrays as a C caller holds them, built once per (cycle, stream slot)
+            for cyc in self.cycles:
+                if cyc.plan is None:
+                    continue
+                offs = cyc.plan.offsets()
+                cyc.arrays = []
+                for slot in range(num_streams):
+                    fb = self.buffers[slot].data_ptr()
+                    in_buf = H._ptr_array([fb + o for o in offs])
+                    tens = H._ptr_array([tensor_ptrs[i] for i in cyc.indices])
+                    outs = H._ptr_array([output_ptrs[i] for i in cyc.indices])
+                    sizes = H._size_array([counts[i] * bs for i in cyc.indices])
+                    cyc.arrays.append((in_buf, tens, outs, sizes, len(cyc.indices)))
         torch.cuda.synchronize()
 
     def reduce_elems(self, cyc, fraction):
@@ -89,14 +120,23 @@ class AllreducePipeline:
             return cyc.buffer_elems
         return reduce_scatter_share(cyc.buffer_elems, int(round(1.0 / fraction)), fused=cyc.plan is not None)
 
-    def run(self, prescale, postscale, peer_ptr=None, num_peers=0, fraction=1.0, kway=True, flags=0):
-        """Queues every cycle; returns without synchronising."""
+    def _copy_arrays(self, out, inp, sizes, n, scale, s):
+        check(lib().hvdhip_batched_scaled_d2d_memcpy(out, inp, sizes, n, float(scale), self.tensor_dtype, s.handle),
+              "hvdhip_batched_scaled_d2d_memcpy")
+
+    def run(self, prescale, postscale, peer_ptr=None, num_peers=0, fraction=1.0, kway=True, flags=0, first_slot=0):
+        """Queues every cycle; returns without synchronising.  Cycle i runs on stream slot
+        (first_slot + i) % streams."""
         for ci, cyc in enumerate(self.cycles):
-            slot = ci % len(self.streams)
+            slot = (first_slot + ci) % len(self.streams)
             s = self.streams[slot]
             if cyc.plan is not None:
                 fb = self.buffers[slot].data_ptr()
-                cyc.plan.pack(fb, prescale, s, flags)
+                if self.array_entry_points:
+                    in_buf, tens, _, sizes, n = cyc.arrays[slot]
+                    self._copy_arrays(in_buf, tens, sizes, n, prescale, s)
+                else:
+                    cyc.plan.pack(fb, prescale, s, flags)
                 res = fb
             else:
                 t, o, n = cyc.single
@@ -113,7 +153,10 @@ class AllreducePipeline:
                 else:
                     for p in ptrs:
                         H.reduce_sum(res, p, n, self.buffer_dtype, s)
-            if cyc.plan is not None:
+            if cyc.plan is not None and self.array_entry_points:
+                in_buf, _, outs, sizes, n = cyc.arrays[slot]
+                self._copy_arrays(outs, in_buf, sizes, n, postscale, s)
+            elif cyc.plan is not None:
                 cyc.plan.unpack(self.buffers[slot].data_ptr(), postscale, s)
             elif postscale != 1.0:
                 t, o, n = cyc.single
