@@ -50,6 +50,21 @@ ROTATE = 6
 # 256 MiB device copy (`bench.py --calibrate`).  The summaries with the commands are the files
 # named here under profiles/; tests/test_host_logic.py re-derives every figure from them.
 TRAFFIC_BYTES_MEASURED = {
+    "c1.pack": 125577703,
+    "c1.reduce": 184760412,
+    "c1.unpack": 125578730,
+    "c2.pack": 93215219,
+    "c2.unpack": 92595010,
+    "c3.pack": 194303412,
+    "c3.reduce": 71756429,
+    "c3.unpack": 197790260,
+    "c4.combine": 677138436,
+    "c4h.combine": 339208460,
+    "c5.pack": 123472076,
+    "c5.reduce": 181653492,
+    "c5.reduce_single": 475145691,
+    "c5.scale_single": 318055994,
+    "c5.unpack": 123477432,
 }
 TRAFFIC_PROFILE = {
     "c1": "profiles/c1_resnet50_fp32_kernels.txt",
@@ -181,11 +196,14 @@ def torch_dtype(dtype):
 
 class Case:
     """One kernel at one grid.  fn() queues one launch on `stream` (the next rotating buffer set
-    every call); alg = algorithmic bytes per launch; kernel = its name as a profiler prints it."""
+    every call); alg = algorithmic bytes per launch; kernel = its name as a profiler prints it
+    (template arguments: ..., 0 pack / 1 unpack, 0 non-temporal / 1 write-through stores).
+    parts: for a call that launches several kernels, [(kernel, algorithmic bytes)] per kernel."""
 
-    def __init__(self, key, kernel, fn, alg, what, workgroups=None, cleanup=None):
+    def __init__(self, key, kernel, fn, alg, what, workgroups=None, cleanup=None, parts=None):
         self.key, self.kernel, self.fn, self.alg, self.what, self.workgroups = key, kernel, fn, alg, what, workgroups
         self.cleanup = cleanup  # destroys the plans behind fn (the closures hold the device memory)
+        self.parts = parts or [(kernel, alg)]
 
 
 def cycle_cases(cfg, counts, tdtype, bdtype, std, peers, share_world, stream, pack_kernel, reduce_kernel,
@@ -259,26 +277,26 @@ def build_cases(cfg):
         counts = [W.numel(x) for x in W.resnet50_shapes()]
         g0 = W.fuse([4 * c for c in counts])[0]
         return cycle_cases("c1", [counts[i] for i in g0], F32, F32, 1e-3, 1, 1, s,
-                           "xfer_k<Scale<float, float>, 0, true>", "reduce_k<float, 1, true>",
-                           "xfer_k<Copy<unsigned int>, 1, false>", 1000)
+                           "xfer_k<Scale<float, float>, 0, 1>", "reduce_k<float, 1, 1>",
+                           "xfer_k<Copy<unsigned int>, 1, 0>", 1000)
     if cfg == "c2":
         counts = W.stress_counts(seed=3)
-        cases = cycle_cases("c2", counts, F32, F32, 1.0, 1, 1, s, "xfer_k<Scale<float, float>, 0, true>",
-                            "reduce_k<float, 1, true>", "xfer_k<Copy<unsigned int>, 1, false>", 2000)
+        cases = cycle_cases("c2", counts, F32, F32, 1.0, 1, 1, s, "xfer_k<Scale<float, float>, 0, 1>",
+                            "reduce_k<float, 1, 1>", "xfer_k<Copy<unsigned int>, 1, 0>", 2000)
         return [cases[0], cases[2]]  # the stress configuration has no reduce stage
     if cfg == "c3":
         counts = [W.numel(x) for x in W.bert_large_shapes()]
         g1 = W.fuse([2 * c for c in counts])[1]
         return cycle_cases("c3", [counts[i] for i in g1], F32, F16, 1e-4, 7, 8, s,
-                           "xfer_k<PackF32F16, 0, true>", "reduce_k<_Float16, 7, true>",
-                           "xfer_k<UnpackF16F32, 1, false>", 3000)
+                           "xfer_k<PackF32F16, 0, 1>", "reduce_k<_Float16, 7, 1>",
+                           "xfer_k<UnpackF16F32, 1, 0>", 3000)
     if cfg == "c5":
         counts = [W.numel(x) for x in W.gpt2_xl_shapes()]
         groups = W.fuse([2 * c for c in counts])
         layer = next(g for g in groups if len(g) == 12)
         cases = cycle_cases("c5", [counts[i] for i in layer], F16, F16, 1e-3, 1, 1, s,
-                            "xfer_k<ScaleHalf, 0, true>", "reduce_k<_Float16, 1, true>",
-                            "xfer_k<Copy<unsigned short>, 1, false>", 5000)
+                            "xfer_k<ScaleHalf, 0, 1>", "reduce_k<_Float16, 1, 1>",
+                            "xfer_k<Copy<unsigned short>, 1, 0>", 5000)
         # the 50257 x 1600 embedding exceeds the threshold and travels alone: prescale tensor -> output,
         # sum in place (ops/nccl_operations.cc:176-186)
         n = counts[0]
@@ -296,10 +314,10 @@ def build_cases(cfg):
             H.reduce_sum(emb[i][1].data_ptr(), emb[i][2].data_ptr(), n, F16, s)
 
         cases += [
-            Case("c5.scale_single", "contig_k<ScaleHalf, false>", scale, 4 * n,
+            Case("c5.scale_single", "contig_k<ScaleHalf, 0>", scale, 4 * n,
                  "the embedding (%d halves) scaled by 0.125 from tensor to output; 3 pairs rotated" % n,
                  (2 * n + 4095) // 4096),
-            Case("c5.reduce_single", "reduce_k<_Float16, 1, true>", reduce_emb, 6 * n,
+            Case("c5.reduce_single", "reduce_k<_Float16, 1, 1>", reduce_emb, 6 * n,
                  "the embedding summed in place with one peer; 3 pairs rotated", (2 * n + 4095) // 4096),
         ]
         return cases
@@ -325,10 +343,11 @@ def build_cases(cfg):
             i = turn[0] = (turn[0] + 1) % len(pairs)
             plan.combine(pairs[i][0].data_ptr(), pairs[i][1].data_ptr(), s)
 
-        return [Case(cfg + ".combine", "dot_partials_k<%s, true> + scaled_add_k<%s, true, false>" % (tname, tname),
-                     combine, 5 * n * es,
+        k1, k2 = "dot_partials_k<%s, true>" % tname, "scaled_add_k<%s, true, 0>" % tname
+        return [Case(cfg + ".combine", k1 + " + " + k2, combine, 5 * n * es,
                      "Adasum combine of two vectors of 2^25 elements in 64 layers: first pass 2 N s bytes (keeps the pair "
-                     "in the Infinity Cache), second pass 3 N s bytes; 4 pairs rotated", None, plan.destroy)]
+                     "in the Infinity Cache), second pass 3 N s bytes; 4 pairs rotated", None, plan.destroy,
+                     parts=[(k1, 2 * n * es), (k2, 3 * n * es)])]
     raise ValueError(cfg)
 
 
@@ -365,7 +384,8 @@ class PipelineRun:
     """A configuration's whole pipeline over `replicas` rotating tensor sets.  All replicas queue on
     the same stream(s) and share the one fusion buffer of each stream slot."""
 
-    def __init__(self, shapes, tdtype, bdtype, std, peers, fraction, streams, replicas, arrays=False):
+    def __init__(self, shapes, tdtype, bdtype, std, peers, fraction, streams, replicas, arrays=False,
+                 completion_events=None):
         import torch
         from horovod_amd import dtype_size, workloads as W
         from horovod_amd.pipeline import AllreducePipeline
@@ -379,7 +399,7 @@ class PipelineRun:
             src = DeviceSet(self.counts, es, lambda n: randn_bytes(n, torch_dtype(tdtype), std, 1 + r))
             dst = DeviceSet(self.counts, es, zeros_bytes)
             pipe = AllreducePipeline(src.ptrs, dst.ptrs, self.counts, tdtype, bdtype, streams=shared, buffers=buffers,
-                                     array_entry_points=arrays)
+                                     array_entry_points=arrays, completion_events=completion_events)
             buffers = pipe.buffers
             bs = dtype_size(pipe.buffer_dtype)
             # one buffer per peer, sized for the largest cycle's reduced chunk, serves every cycle
@@ -678,8 +698,10 @@ def extras(headline_cases_block):
     F32, F16 = DTYPE["float32"], DTYPE["float16"]
     out = {}
 
-    def pipeline(name, shapes, tdt, bdt, std, peers, fraction, streams, replicas, steps, arrays=False, note=None):
-        run = PipelineRun(shapes, tdt, bdt, std, peers, fraction, streams, replicas, arrays=arrays)
+    def pipeline(name, shapes, tdt, bdt, std, peers, fraction, streams, replicas, steps, arrays=False, note=None,
+                 completion_events=None):
+        run = PipelineRun(shapes, tdt, bdt, std, peers, fraction, streams, replicas, arrays=arrays,
+                          completion_events=completion_events)
         sec = timed(run.one_pass, run.sync, steps, max(2, steps // 10))
         out[name] = pipeline_figures(run, sec, streams, note)
         run.destroy()
@@ -705,7 +727,11 @@ def extras(headline_cases_block):
                   "200 repetitions timed; every kernel behind its predecessor on one stream")
     kernels("c2_fusion_stress", "c2")
     pipeline("c2_fusion_stress_two_streams", stress, F32, F32, 1.0, 0, 1.0, 2, 8, 200,
-             note="consecutive repetitions alternate over two stream slots, each with its own fusion buffer")
+             note="consecutive repetitions alternate over two stream slots, each with its own fusion buffer; a pooled "
+                  "completion event behind every repetition, as GPUOpContext::FinalizeGPUQueue records one per response")
+    pipeline("c2_fusion_stress_two_streams_no_completion_events", stress, F32, F32, 1.0, 0, 1.0, 2, 8, 200,
+             completion_events=False,
+             note="the same without the per-repetition completion event (the streams are synchronised at the end)")
     try:
         out["c2_fusion_stress"]["execute_vs_per_tensor_copies"] = per_tensor_comparator()
     except Exception as e:  # pragma: no cover
@@ -774,7 +800,12 @@ def main():
         return
 
     if args.kernel_only:
-        for c in build_cases(args.kernel_only):
+        cases = build_cases(args.kernel_only)
+        # what the launches below are, for whoever reads the profiler's output
+        print("CASES " + json.dumps({"launches_per_case": args.warmup + args.steps,
+                                     "cases": [{"case": c.key, "parts": c.parts, "workgroups": c.workgroups,
+                                                "what": c.what} for c in cases]}), flush=True)
+        for c in cases:
             for _ in range(args.warmup + args.steps):
                 c.fn()
             stream.synchronize()

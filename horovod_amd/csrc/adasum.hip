@@ -190,6 +190,12 @@ struct Axpby {
 };
 // ScaledAddfp16, adasum.h:482-500: float coefficients, t = ca*a rounded to
 // fp32, r = fma(cb, b, t), rounded to half.
+// ScaledAddfp16, adasum.h:482-500: float coefficients, t = ca*a rounded to fp32, r = fma(cb, b, t)
+// rounded to fp32, then to half.  Both fp32 results are kept apart from what follows them: a fused
+// mixed-precision product would take a +0 addend and lose the sign of a -0 product, and a fused
+// fma-and-narrow rounds the exact sum once where fmadd_ps followed by cvtps_ph rounds twice
+// (it differs from the reference in the last bit of some elements).  The widening of b folds
+// into the fma, and pairs of results narrow with one packed conversion.
 template <>
 struct Axpby<half_t> {
   static __device__ __forceinline__ half_t f(double ca, half_t a, double cb, half_t b) {
@@ -370,6 +376,7 @@ namespace {
 // that it is kept: measured on the combine, +28 % at 2 x 16 MiB, +10 % at 2 x 32 MiB,
 // +6 % at 2 x 64 MiB and +2.5 % at 2 x 128 MiB; at 2 x 256 MiB it costs 0.8 % and beyond that nothing is left of it.
 // The largest pair (both vectors, bytes) that is kept:
+// (Loading the kept pass with the sc0 and/or sc1 bits instead of plainly changes nothing.)
 constexpr uint64_t kKeepCachedBytes = (uint64_t)320 << 20;
 
 template <bool KEEP>

@@ -74,7 +74,7 @@ constexpr uint64_t kMaxWorkgroups = 1ull << 23;
 // HVDHIP_CHUNK_BYTES (a multiple of 4096) overrides all three, for tuning.
 enum class Family { kXfer, kXferNarrowing, kReduce, kAdasum };
 constexpr uint32_t kXferChunkBytes = 4096;
-constexpr uint32_t kXferNarrowingChunkBytes = 8192;  // fp32 -> fp16 pack: 8-byte stores per lane
+constexpr uint32_t kXferNarrowingChunkBytes = 8192;  // fp32 -> fp16 pack: 32 bytes in, 16 out per lane
 constexpr uint32_t kReduceChunkBytes = 4096;
 constexpr uint32_t kAdasumChunkBytes = 16384;
 uint32_t chunk_bytes(Family f);

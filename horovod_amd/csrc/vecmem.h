@@ -70,6 +70,13 @@ struct Arr {
 // still be in the Infinity Cache.
 template <typename T, int N, bool NT = true>
 __device__ __forceinline__ Arr<T, N> ldv(gptr<const T> p) {
+  if constexpr (sizeof(T) * N == 32) {  // two 16-byte accesses
+    Arr<T, N> out;
+    const Arr<T, N / 2> lo = ldv<T, N / 2, NT>(p), hi = ldv<T, N / 2, NT>(p + N / 2);
+    __builtin_memcpy(out.v, lo.v, 16);
+    __builtin_memcpy(out.v + N / 2, hi.v, 16);
+    return out;
+  } else {
   typedef typename Raw<(int)sizeof(T) * N, (int)alignof(T)>::type R;
   typename RawSel<(int)sizeof(T) * N>::type r;
   if constexpr (NT && HVDHIP_NONTEMPORAL) {
@@ -78,6 +85,7 @@ __device__ __forceinline__ Arr<T, N> ldv(gptr<const T> p) {
     r = *reinterpret_cast<gptr<const R>>(p);
   }
   return __builtin_bit_cast(Arr<T, N>, r);
+  }
 }
 
 template <typename T, int N>
@@ -150,7 +158,13 @@ __device__ __forceinline__ Window store_window(gptr<T> base, uint32_t bytes) {
 // Stores N elements of T at byte offset `off` of the window.
 template <int ST, typename T, int N>
 __device__ __forceinline__ void stw(const Window& w, uint32_t off, const Arr<T, N>& a) {
-  if constexpr (ST == kStoreWT) {
+  if constexpr (sizeof(T) * N == 32) {  // two 16-byte accesses
+    Arr<T, N / 2> lo, hi;
+    __builtin_memcpy(lo.v, a.v, 16);
+    __builtin_memcpy(hi.v, a.v + N / 2, 16);
+    stw<ST, T, N / 2>(w, off, lo);
+    stw<ST, T, N / 2>(w, off + 16, hi);
+  } else if constexpr (ST == kStoreWT) {
     typedef typename RawSel<(int)sizeof(T) * N>::type R;
 #ifndef HVDHIP_WT_AUX
 #define HVDHIP_WT_AUX (1 | 16)  // sc0 | sc1

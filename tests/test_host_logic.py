@@ -32,3 +32,45 @@ def test_bert_large_cycles_reduce_an_eighth():
         n = sum((2 * counts[i] + 15) // 16 * 16 for i in g) // 2  # padded fp16 elements of the cycle
         per = W.reduce_scatter_share(n, 8)
         assert 0 <= per - n / 8 < 64
+
+
+def _profile_rows(path):
+    """(factors, rows) of a kernel summary under profiles/: the calibration factors and the table."""
+    import re
+    text = open(os.path.join(ROOT, path)).read()
+    m = re.search(r"calibration factors: FETCH_SIZE x ([0-9.]+)\s+WRITE_SIZE x ([0-9.]+)", text)
+    factors = (float(m.group(1)), float(m.group(2)))
+    lines = text.splitlines()
+    head = next(i for i, l in enumerate(lines) if l.startswith("case | kernel |"))
+    cols = [c.strip() for c in lines[head].split("|")]
+    rows = []
+    for l in lines[head + 1:]:
+        if "|" not in l:
+            break
+        rows.append(dict(zip(cols, [c.strip() for c in l.split("|")])))
+    return factors, rows
+
+
+def test_traffic_constants_of_the_bench_follow_from_the_profiles():
+    """bench.py reports `roofline.traffic` from constants measured once with rocprofv3; each must be
+    what the committed summary's own counter averages and calibration factors give."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_module", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    seen = {}
+    for cfg, path in bench.TRAFFIC_PROFILE.items():
+        (ff, wf), rows = _profile_rows(path)
+        assert 1.5 < ff < 2.5 and 0.95 < wf < 1.05
+        for r in rows:
+            read_b = float(r["FETCH_KiB"]) * 1024 * ff
+            written_b = float(r["WRITE_KiB"]) * 1024 * wf
+            assert abs(read_b - int(r["read_B"])) <= 1 and abs(written_b - int(r["written_B"])) <= 1, r
+            assert abs(read_b + written_b - int(r["traffic_B"])) <= 1, r
+            alg = int(r["algorithmic_B"])
+            assert abs(int(r["traffic_B"]) / alg - float(r["traffic/algorithmic"])) < 1e-3
+            assert abs(alg / float(r["avg_ns"]) / 8000.0 - float(r["frac"])) < 1e-4
+            # nothing is re-read: traffic within 4 % of the algorithmic bytes
+            assert 0.96 < int(r["traffic_B"]) / alg < 1.04, r
+            seen[r["case"]] = seen.get(r["case"], 0) + int(r["traffic_B"])
+    assert seen == bench.TRAFFIC_BYTES_MEASURED

@@ -95,13 +95,12 @@ def test_streaming_stores_carry_one_of_the_two_policies(kernels):
     for name, lines in kernels.items():
         if "finalize_k" in name or "one_layer_tables_k" in name:
             continue  # stores a layer's sums and coefficients, or a chunk table: nothing streamed
-        streams_halves = "PackF32F16" in name  # the narrowing pack stores 8 bytes per lane
         # sums and coefficients of a layer or chunk, written by one lane
         small_results = 4 if ("scaled_add_k" in name or "dot_partials_k" in name) else 0
         plain = 0
         for ins in lines:
             op = ins.split()[0]
-            if op == "global_store_dwordx4" or (streams_halves and op == "global_store_dwordx2"):
+            if op == "global_store_dwordx4":
                 checked += 1
                 plain += " nt" not in ins
             elif op in ("buffer_store_dwordx4", "buffer_store_dwordx2"):
