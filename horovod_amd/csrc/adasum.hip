@@ -33,9 +33,11 @@ namespace hvdhip {
 namespace {
 
 // Chunk table entry as used here: tensor = index of the chunk's first element
-// in the vectors, output = layer number, off = the chunk's number in layer order
-// (the slot of its partial triple; the table itself is in XCD order), n = elements
-// in the chunk.
+// in the vectors, output = layer number in the low and the layer's first partial
+// triple in the high 32 bits, off = the chunk's number in layer order (the slot of
+// its partial triple; the table itself is in XCD order), n = elements in the chunk,
+// pad = number of partial triples of the layer.  With its layer's entry folded in,
+// a workgroup needs no second dependent load to find its layer's partial sums.
 //
 // Layer table entry: first partial triple of the layer and how many it has.
 struct Layer {
@@ -231,19 +233,18 @@ __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ ch
   const Window out = store_window<ST>(pa, n * (uint32_t)sizeof(T));
   uint32_t v = threadIdx.x;
   double ca, cb;
+  const uint32_t layer = (uint32_t)c.output;
   if (FUSED) {
-    const Layer L = layers[c.output];
-    // this lane's share of the layer's triples first, the data loads behind them: loads return
-    // in order, so the sums below wait for the triples only
-    Triple t0 = {0., 0., 0.}, t1 = {0., 0., 0.};
-    if (threadIdx.x < L.count) {
-      const uint64_t i = 3 * ((uint64_t)L.first + threadIdx.x);
-      t0 = Triple{partials[i], partials[i + 1], partials[i + 2]};
-    }
-    if (threadIdx.x + kWG < L.count) {
-      const uint64_t i = 3 * ((uint64_t)L.first + threadIdx.x + kWG);
-      t1 = Triple{partials[i], partials[i + 1], partials[i + 2]};
-    }
+    const Layer L = {(uint32_t)(c.output >> 32), c.pad};
+    // this lane's share of the layer's triples first, the data loads right behind them: loads
+    // return in order, so the sums below wait for the triples only.  The triple loads are
+    // unconditional (a lane beyond the layer's count re-reads the last triple and drops it), so
+    // that nothing waits for them before the data loads are out.
+    const uint32_t last = L.count - 1;  // a chunk's layer has at least this chunk's triple
+    const uint64_t i0 = 3 * ((uint64_t)L.first + (threadIdx.x < last ? threadIdx.x : last));
+    const uint64_t i1 = 3 * ((uint64_t)L.first + (threadIdx.x + kWG < last ? threadIdx.x + kWG : last));
+    const Triple r0 = {partials[i0], partials[i0 + 1], partials[i0 + 2]};
+    const Triple r1 = {partials[i1], partials[i1 + 1], partials[i1 + 2]};
     const bool full = v + (kUnroll - 1) * kWG < nv;
     V x[kUnroll], y[kUnroll];
     if (full) {
@@ -253,6 +254,9 @@ __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ ch
         y[u] = ldv<T, VEC>(pb + (size_t)(v + u * kWG) * VEC);
       }
     }
+    const bool in0 = threadIdx.x < L.count, in1 = threadIdx.x + kWG < L.count;
+    const Triple t0 = {in0 ? r0.d : 0., in0 ? r0.a : 0., in0 ? r0.b : 0.};
+    const Triple t1 = {in1 ? r1.d : 0., in1 ? r1.a : 0., in1 ? r1.b : 0.};
     Triple t = {0., 0., 0.};
     t.d += t0.d; t.a += t0.a; t.b += t0.b;  // the order of finalize_k: i = lane, lane + kWG
     t.d += t1.d; t.a += t1.a; t.b += t1.b;
@@ -263,11 +267,11 @@ __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ ch
       cc[0] = ca;
       cc[1] = cb;
       if (c.off == L.first) {
-        normdots[3 * c.output + 0] = r.d;
-        normdots[3 * c.output + 1] = r.a;
-        normdots[3 * c.output + 2] = r.b;
-        coeffs_out[2 * c.output + 0] = ca;
-        coeffs_out[2 * c.output + 1] = cb;
+        normdots[3 * (uint64_t)layer + 0] = r.d;
+        normdots[3 * (uint64_t)layer + 1] = r.a;
+        normdots[3 * (uint64_t)layer + 2] = r.b;
+        coeffs_out[2 * (uint64_t)layer + 0] = ca;
+        coeffs_out[2 * (uint64_t)layer + 1] = cb;
       }
     }
     if (blockIdx.x == 0) {
@@ -296,8 +300,8 @@ __global__ __launch_bounds__(kWG) void scaled_add_k(const Chunk* __restrict__ ch
     }
   } else {
     // coeffs == nullptr: every layer uses the by-value pair (ca_arg, cb_arg).
-    ca = coeffs ? coeffs[2 * c.output] : ca_arg;
-    cb = coeffs ? coeffs[2 * c.output + 1] : cb_arg;
+    ca = coeffs ? coeffs[2 * (uint64_t)layer] : ca_arg;
+    cb = coeffs ? coeffs[2 * (uint64_t)layer + 1] : cb_arg;
   }
   for (; v + (kUnroll - 1) * kWG < nv; v += kUnroll * kWG) {
     V x[kUnroll], y[kUnroll];
@@ -337,7 +341,7 @@ __global__ __launch_bounds__(kWG) void one_layer_tables_k(Chunk* __restrict__ ch
   const uint64_t start = (uint64_t)c * chunk_units;
   const uint64_t left = count - start;
   chunks[xcd_slot(c, nchunks, run)] =
-      Chunk{start, 0, (uint64_t)c, (uint32_t)(left < chunk_units ? left : chunk_units), 0};
+      Chunk{start, 0, (uint64_t)c, (uint32_t)(left < chunk_units ? left : chunk_units), nchunks};
 }
 
 // Scratch of hvdhip_adasum_combine_static: the tables and partial sums that a plan would hold in
@@ -560,6 +564,10 @@ int hvdhip_adasum_plan_create(const int* tensor_counts, int nlayers, int dtype,
                              (uint32_t)(left < chunk_units ? left : chunk_units), 0});
     }
     layers[(size_t)i].count = (uint32_t)chunks.size() - layers[(size_t)i].first;
+    for (size_t c = layers[(size_t)i].first; c < chunks.size(); ++c) {  // the layer's entry, folded into its chunks
+      chunks[c].output |= (uint64_t)layers[(size_t)i].first << 32;
+      chunks[c].pad = layers[(size_t)i].count;
+    }
     if (layers[(size_t)i].count > max_layer_chunks) max_layer_chunks = layers[(size_t)i].count;
     if (chunks.size() > kMaxWorkgroups) return fail(HVDHIP_ERR_TOO_LARGE, "the vectors need more than 2^23 workgroups");
     off += n;
