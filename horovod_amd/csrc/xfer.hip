@@ -218,11 +218,13 @@ __global__ __launch_bounds__(kWG) void contig_k(const typename Op::S* src, typen
 // Host side
 // ----------------------------------------------------------------------
 
+// gathers: a direct transfer whose destinations lie back to back, i.e. a pack into a fusion buffer
+// through the array-taking entry points; it stores like a pack.
 template <class Op, int MODE>
-int launch_xfer(const DevTables& t, uint64_t base, typename Op::P p, hipStream_t stream) {
+int launch_xfer(const DevTables& t, uint64_t base, typename Op::P p, hipStream_t stream, bool gathers = false) {
   if (t.nchunks == 0) return 0;
   constexpr bool converting = sizeof(typename Op::S) != sizeof(typename Op::D);
-  const Stores family = MODE == kDirect ? Stores::kDirect
+  const Stores family = MODE == kDirect ? (gathers ? Stores::kPack : Stores::kDirect)
                         : MODE == kPack ? (converting ? Stores::kPackNarrowing : Stores::kPack)
                                         : (converting ? Stores::kUnpackWidening : Stores::kUnpack);
   with_store_policy(family, [&](auto st) {
@@ -236,24 +238,24 @@ int launch_xfer(const DevTables& t, uint64_t base, typename Op::P p, hipStream_t
 // dtype.  scale == 1.0 is a plain copy, valid for every dtype.
 template <int MODE>
 int launch_same_dtype(const DevTables& t, uint64_t base, double scale, int dtype,
-                      hipStream_t stream) {
+                      hipStream_t stream, bool gathers = false) {
   if (scale == 1.0) {
     switch (dtype_size(dtype)) {
-    case 1: return launch_xfer<Copy<uint8_t>, MODE>(t, base, {}, stream);
-    case 2: return launch_xfer<Copy<uint16_t>, MODE>(t, base, {}, stream);
-    case 4: return launch_xfer<Copy<uint32_t>, MODE>(t, base, {}, stream);
-    case 8: return launch_xfer<Copy<uint64_t>, MODE>(t, base, {}, stream);
+    case 1: return launch_xfer<Copy<uint8_t>, MODE>(t, base, {}, stream, gathers);
+    case 2: return launch_xfer<Copy<uint16_t>, MODE>(t, base, {}, stream, gathers);
+    case 4: return launch_xfer<Copy<uint32_t>, MODE>(t, base, {}, stream, gathers);
+    case 8: return launch_xfer<Copy<uint64_t>, MODE>(t, base, {}, stream, gathers);
     default: return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE, "unknown dtype %d", dtype);
     }
   }
   switch (dtype) {
-  case HVDHIP_UINT8: return launch_xfer<Scale<uint8_t, double>, MODE>(t, base, {scale}, stream);
-  case HVDHIP_INT8: return launch_xfer<Scale<int8_t, double>, MODE>(t, base, {scale}, stream);
-  case HVDHIP_INT32: return launch_xfer<Scale<int32_t, double>, MODE>(t, base, {scale}, stream);
-  case HVDHIP_INT64: return launch_xfer<Scale<int64_t, double>, MODE>(t, base, {scale}, stream);
-  case HVDHIP_FLOAT16: return launch_xfer<ScaleHalf, MODE>(t, base, {fp16_scale_factor(scale)}, stream);
-  case HVDHIP_FLOAT32: return launch_xfer<Scale<float, float>, MODE>(t, base, {(float)scale}, stream);
-  case HVDHIP_FLOAT64: return launch_xfer<Scale<double, double>, MODE>(t, base, {scale}, stream);
+  case HVDHIP_UINT8: return launch_xfer<Scale<uint8_t, double>, MODE>(t, base, {scale}, stream, gathers);
+  case HVDHIP_INT8: return launch_xfer<Scale<int8_t, double>, MODE>(t, base, {scale}, stream, gathers);
+  case HVDHIP_INT32: return launch_xfer<Scale<int32_t, double>, MODE>(t, base, {scale}, stream, gathers);
+  case HVDHIP_INT64: return launch_xfer<Scale<int64_t, double>, MODE>(t, base, {scale}, stream, gathers);
+  case HVDHIP_FLOAT16: return launch_xfer<ScaleHalf, MODE>(t, base, {fp16_scale_factor(scale)}, stream, gathers);
+  case HVDHIP_FLOAT32: return launch_xfer<Scale<float, float>, MODE>(t, base, {(float)scale}, stream, gathers);
+  case HVDHIP_FLOAT64: return launch_xfer<Scale<double, double>, MODE>(t, base, {scale}, stream, gathers);
   default:
     return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE, "dtype %d cannot be scaled by a factor other than 1", dtype);
   }
@@ -324,6 +326,10 @@ struct CachedCopy {
   bool upload_complete = false;     // `uploaded` has been seen complete: other streams need not wait for it
   hipStream_t build_stream = nullptr;
   std::vector<hipStream_t> streams;  // every stream that holds, or held, a launch reading the table
+  // The destinations lie back to back (each starts within 16 bytes after the one before ends) and
+  // there are several: the caller packs into a fusion buffer, which the next kernel on the stream
+  // reads, so the copy stores like a pack (through the Infinity Cache).
+  bool gathers = false;
 };
 
 // Buffers of an evicted entry; free for reuse once every event has completed.
@@ -572,6 +578,11 @@ int cached_tables(CopyCache& c, void* const* out, const void* const* in, const s
   entry.tables.chunks = static_cast<Chunk*>(entry.buf.dev);
   entry.tables.nchunks = (uint32_t)nchunks;
   entry.build_stream = stream;
+  entry.gathers = n > 1;
+  for (int i = 0; i + 1 < n && entry.gathers; ++i) {
+    const uint64_t end = (uint64_t)(uintptr_t)out[i] + sizes[i], next = (uint64_t)(uintptr_t)out[i + 1];
+    entry.gathers = next >= end && next - end < 16;
+  }
   c.bytes += entry.buf.cap;
   c.lru.push_front(std::move(entry));
   c.index.emplace(hash, c.lru.begin());
@@ -650,7 +661,7 @@ int hvdhip_batched_d2d_memcpy(void* const* out, const void* const* in, const siz
   rc = cached_tables(*cache, out, in, sizes, num_copies, 1, s, &entry);
   if (rc) return rc;
   mark_used(entry, s);
-  rc = launch_xfer<Copy<uint8_t>, kDirect>(entry->tables, 0, {}, s);
+  rc = launch_xfer<Copy<uint8_t>, kDirect>(entry->tables, 0, {}, s, entry->gathers);
   return rc ? rc : ok();
 }
 
@@ -678,7 +689,7 @@ int hvdhip_batched_scaled_d2d_memcpy(void* const* out, const void* const* in,
   rc = cached_tables(*cache, out, in, sizes, num_copies, es, s, &entry);
   if (rc) return rc;
   mark_used(entry, s);
-  rc = launch_same_dtype<kDirect>(entry->tables, 0, scale_factor, dtype, s);
+  rc = launch_same_dtype<kDirect>(entry->tables, 0, scale_factor, dtype, s, entry->gathers);
   return rc ? rc : ok();
 }
 

@@ -171,6 +171,9 @@ int hvdhip_timer_destroy(void* timer);
  * the same arrays are seen again (one table per distinct set of copies, as many
  * as the job cycles through); the first call with a new set stages its table with
  * an asynchronous copy on the same stream and does not wait for the device.
+ * When the destinations lie back to back (each begins within 16 bytes after the
+ * one before ends: a pack into a fusion buffer) the copy writes through the
+ * Infinity Cache as hvdhip_fusion_pack does; otherwise it stores past it.
  * A stream that these entry points have used must be idle when it is destroyed
  * (hvdhip_stream_destroy sees to that itself). */
 int hvdhip_batched_d2d_memcpy(void* const* out, const void* const* in, const size_t* sizes,
