@@ -76,6 +76,30 @@ def test_c1_resnet50_fp32_pack_prescale_sum_unpack(gpu, orc):
     pipe.destroy()
 
 
+def test_c1_through_the_array_taking_entry_points(gpu, orc):
+    """The same configuration with every pack and unpack through hvdhip_batched_scaled_d2d_memcpy (the launcher
+    that takes the copies as arrays, ops/gpu_operations.cc:186-206) on two stream slots: the pack's destinations
+    lie back to back, which the library recognises and stores like a pack; results equal the oracle's."""
+    from horovod_amd import workloads as W
+    from horovod_amd.pipeline import AllreducePipeline
+    counts = [W.numel(s) for s in W.resnet50_shapes()]
+    rng, prng = np.random.default_rng(1), np.random.default_rng(2)
+    offs, img, vals = _host_set(counts, 4, lambda n: (rng.standard_normal(n) * 1e-3).astype(np.float32))
+    d_in = torch.from_numpy(img).cuda()
+    d_out = torch.zeros_like(d_in)
+    pipe = AllreducePipeline([d_in.data_ptr() + o for o in offs], [d_out.data_ptr() + o for o in offs], counts, F32,
+                             num_streams=2, array_entry_points=True)
+    peers, peer_vals = _peer_images(pipe, counts, 4, lambda n: (prng.standard_normal(n) * 1e-3).astype(np.float32))
+    for rep in range(2):  # the second pass finds its copy tables in the cache
+        pipe.run(0.125, 0.5, lambda ci, p: peers[ci].data_ptr(), 1)
+        pipe.synchronize()
+    out = d_out.cpu().numpy()
+    for i, (o, c, v) in enumerate(zip(offs, counts, vals)):
+        want = orc.scale_buffer(orc.sum(peer_vals[i], orc.scale_buffer(v, 0.125, F32), F32), 0.5, F32)
+        assert np.array_equal(out[o:o + 4 * c].view(np.uint32), want.view(np.uint32)), "tensor %d" % i
+    pipe.destroy()
+
+
 def test_c2_fusion_stress_pack_unpack(gpu, orc):
     from horovod_amd import workloads as W
     from horovod_amd.pipeline import AllreducePipeline
