@@ -8,7 +8,7 @@
 //
 // Pass 1 (dot_partials_k): one workgroup per chunk of a layer.  Each lane
 // streams 16-byte pieces of a and b, widens to double and keeps two
-// independent fma chains per sum; lanes combine with wave64 shuffles, the four
+// independent fma chains per sum; lanes combine with wave64 DPP adds, the four
 // wavefronts through LDS, and the workgroup writes one {dot, |a|^2, |b|^2}
 // triple.  Pass 1b (finalize_k): one workgroup per layer adds that layer's
 // triples in a fixed order and evaluates the coefficients.  No floating-point
@@ -49,17 +49,39 @@ struct Triple {
   double d, a, b;
 };
 
+// x + (x of the lane that the DPP control CTRL names), for the rows in ROW_MASK; lanes without a
+// source (or outside the mask) add zero.  Two 32-bit DPP moves and one add: data-parallel
+// primitives move data between lanes inside the vector ALU, where a shuffle goes through the LDS
+// crossbar and costs a memory-pipeline round trip per step.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_add(double x) {
+  const int lo = __double2loint(x), hi = __double2hiint(x);
+  const int lo2 = __builtin_amdgcn_update_dpp(0, lo, CTRL, ROW_MASK, 0xf, false);
+  const int hi2 = __builtin_amdgcn_update_dpp(0, hi, CTRL, ROW_MASK, 0xf, false);
+  return x + __hiloint2double(hi2, lo2);
+}
+
+// Sum over the 64 lanes of a wavefront in a fixed order; the total arrives in lane 63.  Within
+// each row of 16 lanes a shifted-add scan (by 1, 2, 4, 8), then lane 15 of rows 0 and 2 into rows
+// 1 and 3, then lane 31 into rows 2 and 3.
+__device__ __forceinline__ double wave_sum(double x) {
+  x = dpp_add<0x111, 0xf>(x);  // row_shr:1
+  x = dpp_add<0x112, 0xf>(x);  // row_shr:2
+  x = dpp_add<0x114, 0xf>(x);  // row_shr:4
+  x = dpp_add<0x118, 0xf>(x);  // row_shr:8
+  x = dpp_add<0x142, 0xa>(x);  // row_bcast:15 into rows 1 and 3
+  x = dpp_add<0x143, 0xc>(x);  // row_bcast:31 into rows 2 and 3
+  return x;
+}
+
 __device__ __forceinline__ Triple wg_reduce(Triple t) {
-  // wave64 tree, then the four wavefronts in order through LDS
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    t.d += __shfl_down(t.d, o, 64);
-    t.a += __shfl_down(t.a, o, 64);
-    t.b += __shfl_down(t.b, o, 64);
-  }
+  // wave64 sums, then the four wavefronts in order through LDS
+  t.d = wave_sum(t.d);
+  t.a = wave_sum(t.a);
+  t.b = wave_sum(t.b);
   __shared__ double red[3][kWG / 64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  if (lane == 0) {
+  if (lane == 63) {
     red[0][wave] = t.d;
     red[1][wave] = t.a;
     red[2][wave] = t.b;
