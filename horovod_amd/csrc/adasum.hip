@@ -101,9 +101,9 @@ __device__ __forceinline__ Triple wg_reduce(Triple t) {
 
 constexpr int kUnroll = 4;
 
-// KEEP: the loads leave the vectors in the Infinity Cache for the scaled add that follows
-// (chosen by the host when both vectors fit there with room to spare).
-template <typename T, bool KEEP>
+// KEEP: which vectors the loads leave in the Infinity Cache for the scaled add that follows
+// (1 a, 2 a and b; chosen by the host by what fits there).
+template <typename T, int KEEP>
 __global__ __launch_bounds__(kWG) void dot_partials_k(const Chunk* __restrict__ chunks,
                                                       const T* __restrict__ a,
                                                       const T* __restrict__ b,
@@ -121,8 +121,8 @@ __global__ __launch_bounds__(kWG) void dot_partials_k(const Chunk* __restrict__ 
     V x[kUnroll], y[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-      x[u] = ldv<T, VEC, !KEEP>(pa + (size_t)(v + u * kWG) * VEC);
-      y[u] = ldv<T, VEC, !KEEP>(pb + (size_t)(v + u * kWG) * VEC);
+      x[u] = ldv<T, VEC, false>(pa + (size_t)(v + u * kWG) * VEC);
+      y[u] = ldv<T, VEC, KEEP != 2>(pb + (size_t)(v + u * kWG) * VEC);
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
@@ -142,7 +142,7 @@ __global__ __launch_bounds__(kWG) void dot_partials_k(const Chunk* __restrict__ 
     }
   }
   for (; v < nv; v += kWG) {
-    const V x = ldv<T, VEC, !KEEP>(pa + (size_t)v * VEC), y = ldv<T, VEC, !KEEP>(pb + (size_t)v * VEC);
+    const V x = ldv<T, VEC, false>(pa + (size_t)v * VEC), y = ldv<T, VEC, KEEP != 2>(pb + (size_t)v * VEC);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
       const double p = (double)x.v[j], q = (double)y.v[j];
@@ -397,15 +397,19 @@ struct hvdhip_adasum_plan {
 
 namespace {
 
-// The scaled add reads both vectors a second time.  When the pair is small enough to still be in
-// the 256 MB Infinity Cache by then, the first pass loads it without the non-temporal hint so
-// that it is kept: measured on the combine, +28 % at 2 x 16 MiB, +10 % at 2 x 32 MiB,
-// +6 % at 2 x 64 MiB and +2.5 % at 2 x 128 MiB; at 2 x 256 MiB it costs 0.8 % and beyond that nothing is left of it.
-// The largest pair (both vectors, bytes) that is kept:
-// (Loading the kept pass with the sc0 and/or sc1 bits instead of plainly changes nothing.)
-constexpr uint64_t kKeepCachedBytes = (uint64_t)320 << 20;
+// The scaled add reads both vectors a second time, and the first pass decides with its loads what
+// the 256 MB Infinity Cache holds by then: loads without the non-temporal hint leave their lines
+// there.  Measured on the combine of fp32 vectors in 64 layers (neither / a alone / both kept):
+//   2 x  32 MiB: 29.0 / 25.9 / 24.7 us      2 x 128 MiB: 103.8 /  96.7 / 100.7 us
+//   2 x  64 MiB: 54.0 / 49.6 / 49.7 us      2 x 192 MiB: 152.2 / 145.6 / 150.1 us
+//   2 x  96 MiB: 79.2 / 73.6 / 75.5 us      2 x 384 MiB: 304.2 / 291.5 / 305.1 us
+// Keeping both pays while the pair fits the cache with room to spare; keeping a alone (the vector
+// that the second pass also rewrites) pays at every size beyond, even where a by itself exceeds
+// the cache, and a pair that fills the cache to the brim (2 x 128 MiB) thrashes when both are kept.
+constexpr uint64_t kKeepBothBytes = (uint64_t)160 << 20;  // largest pair (both vectors) kept whole
+inline int keep_mode(uint64_t vector_bytes) { return 2 * vector_bytes <= kKeepBothBytes ? 2 : 1; }
 
-template <bool KEEP>
+template <int KEEP>
 void launch_dot_partials(hvdhip_adasum_plan* p, const void* a, const void* b, hipStream_t s) {
   const DevTables& t = p->tables;
   switch (p->dtype) {
@@ -430,10 +434,10 @@ int plan_dot_norms(hvdhip_adasum_plan* p, const void* a, const void* b, hipStrea
   if (p->nlayers == 0) return 0;
   const DevTables& t = p->tables;
   if (t.nchunks > 0) {
-    if (2 * (uint64_t)p->total * (uint64_t)dtype_size(p->dtype) <= kKeepCachedBytes)
-      launch_dot_partials<true>(p, a, b, s);
+    if (keep_mode((uint64_t)p->total * (uint64_t)dtype_size(p->dtype)) == 2)
+      launch_dot_partials<2>(p, a, b, s);
     else
-      launch_dot_partials<false>(p, a, b, s);
+      launch_dot_partials<1>(p, a, b, s);
     HVDHIP_CHECK_LAUNCH("dot_partials_k");
   }
   if (!finalize) return 0;
