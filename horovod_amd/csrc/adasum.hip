@@ -403,9 +403,10 @@ namespace {
 //   2 x  32 MiB: 29.0 / 25.9 / 24.7 us      2 x 128 MiB: 103.8 /  96.7 / 100.7 us
 //   2 x  64 MiB: 54.0 / 49.6 / 49.7 us      2 x 192 MiB: 152.2 / 145.6 / 150.1 us
 //   2 x  96 MiB: 79.2 / 73.6 / 75.5 us      2 x 384 MiB: 304.2 / 291.5 / 305.1 us
-// Keeping both pays while the pair fits the cache with room to spare; keeping a alone (the vector
-// that the second pass also rewrites) pays at every size beyond, even where a by itself exceeds
-// the cache, and a pair that fills the cache to the brim (2 x 128 MiB) thrashes when both are kept.
+// Keeping both pays while the pair fits the cache with room to spare; keeping one of the two pays
+// at every size beyond, even where one vector by itself exceeds the cache (keeping b instead of a
+// measures the same), and a pair that fills the cache to the brim (2 x 128 MiB) thrashes when both
+// are kept.
 constexpr uint64_t kKeepBothBytes = (uint64_t)160 << 20;  // largest pair (both vectors) kept whole
 inline int keep_mode(uint64_t vector_bytes) { return 2 * vector_bytes <= kKeepBothBytes ? 2 : 1; }
 
