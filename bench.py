@@ -50,21 +50,21 @@ ROTATE = 6
 # 256 MiB device copy (`bench.py --calibrate`).  The summaries with the commands are the files
 # named here under profiles/; tests/test_host_logic.py re-derives every figure from them.
 TRAFFIC_BYTES_MEASURED = {
-    "c1.pack": 125571719,
+    "c1.pack": 125571679,
     "c1.reduce": 184760412,
-    "c1.unpack": 125582334,
-    "c2.pack": 93207974,
-    "c2.unpack": 92592105,
-    "c3.pack": 194430415,
-    "c3.reduce": 71756289,
-    "c3.unpack": 197788736,
-    "c4.combine": 669871672,
-    "c4h.combine": 336619439,
-    "c5.pack": 123465031,
+    "c1.unpack": 125581985,
+    "c2.pack": 93208344,
+    "c2.unpack": 92593204,
+    "c3.pack": 194434537,
+    "c3.reduce": 71756449,
+    "c3.unpack": 197803761,
+    "c4.combine": 670862926,
+    "c4h.combine": 336545337,
+    "c5.pack": 123465011,
     "c5.reduce": 181653492,
     "c5.reduce_single": 475145691,
-    "c5.scale_single": 318070503,
-    "c5.unpack": 123487764,
+    "c5.scale_single": 318074457,
+    "c5.unpack": 123480144,
 }
 TRAFFIC_PROFILE = {
     "c1": "profiles/c1_resnet50_fp32_kernels.txt",
