@@ -183,7 +183,26 @@ __global__ __launch_bounds__(kWG) void finalize_k(const Layer* __restrict__ laye
   const Layer L = layers[blockIdx.x];
   const uint64_t first = L.first, count = L.count;
   Triple t = {0., 0., 0.};
-  for (uint64_t i = threadIdx.x; i < count; i += kWG) {
+  // A lane adds triples lane, lane + kWG, lane + 2 kWG ... in that order; eight are fetched at a
+  // time so that a layer of thousands of chunks (one workgroup reads them all) does not pay one
+  // memory round trip per step.
+  constexpr int kAhead = 8;
+  uint64_t i = threadIdx.x;
+  for (; i + (kAhead - 1) * kWG < count; i += kAhead * kWG) {
+    double v[kAhead][3];
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+#pragma unroll
+      for (int j = 0; j < 3; ++j) v[u][j] = partials[3 * (first + i + (uint64_t)u * kWG) + j];
+    }
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      t.d += v[u][0];
+      t.a += v[u][1];
+      t.b += v[u][2];
+    }
+  }
+  for (; i < count; i += kWG) {
     t.d += partials[3 * (first + i) + 0];
     t.a += partials[3 * (first + i) + 1];
     t.b += partials[3 * (first + i) + 2];
@@ -585,10 +604,18 @@ int hvdhip_adasum_plan_create(const int* tensor_counts, int nlayers, int dtype,
     if (tensor_counts[i] < 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "tensor_counts[%d] is negative", i);
     const uint64_t n = (uint64_t)tensor_counts[i];
     layers[(size_t)i].first = (uint32_t)chunks.size();
-    for (uint64_t start = 0; start < n; start += chunk_units) {
+    // Chunks are cut at multiples of the chunk size counted from the start of the vectors, not of
+    // the layer: a layer begins wherever the one before it ends, and a chunk that starts in the
+    // middle of a 16-byte piece (let alone of a cache line) makes every load of its workgroup
+    // straddle two.  So a layer's first chunk runs up to the next such boundary, and all its
+    // other chunks start on one.
+    uint64_t start = 0;
+    while (start < n) {
+      const uint64_t to_boundary = chunk_units - (off + start) % chunk_units;
       const uint64_t left = n - start;
-      chunks.push_back(Chunk{off + start, (uint64_t)i, (uint64_t)chunks.size(),
-                             (uint32_t)(left < chunk_units ? left : chunk_units), 0});
+      const uint64_t len = left < to_boundary ? left : to_boundary;
+      chunks.push_back(Chunk{off + start, (uint64_t)i, (uint64_t)chunks.size(), (uint32_t)len, 0});
+      start += len;
     }
     layers[(size_t)i].count = (uint32_t)chunks.size() - layers[(size_t)i].first;
     for (size_t c = layers[(size_t)i].first; c < chunks.size(); ++c) {  // the layer's entry, folded into its chunks
