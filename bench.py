@@ -58,8 +58,8 @@ TRAFFIC_BYTES_MEASURED = {
     "c3.pack": 194434537,
     "c3.reduce": 71756449,
     "c3.unpack": 197803761,
-    "c4.combine": 670862926,
-    "c4h.combine": 336545337,
+    "c4.combine": 662271124,
+    "c4h.combine": 331107195,
     "c5.pack": 123465011,
     "c5.reduce": 181653492,
     "c5.reduce_single": 475145691,
