@@ -461,7 +461,10 @@ int evict_one(CopyCache& c) {
   for (hipStream_t s : victim->streams) {
     hipEvent_t e = nullptr;
     int rc = order_event(c, &e);
-    if (rc) return rc;
+    if (rc) {  // the victim stays; the events taken so far go back (recording them again later is fine)
+      for (hipEvent_t taken : r.events) c.idle_events.push_back(taken);
+      return rc;
+    }
     if (hipEventRecord(e, s) == hipSuccess) {
       r.events.push_back(e);
     } else {
