@@ -720,6 +720,10 @@ def extras(headline_cases_block):
     # C1 on two streams (the headline is the one-stream figure); its kernel blocks come from the headline
     pipeline("c1_resnet50_fp32_two_streams", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0, 2, 4, 200)
     out["c1_resnet50_fp32_two_streams"]["kernels"] = headline_cases_block
+    pipeline("c1_resnet50_fp32_one_stream_completion_events", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0, 1, 4, 200,
+             completion_events=True,
+             note="the headline pipeline with a pooled completion event recorded behind every cycle and waited for by "
+                  "the host, as GPUOpContext::FinalizeGPUQueue does once per response (ops/gpu_operations.cc:50-98)")
 
     # C2: fusion stress, pack + unpack, 200 repetitions
     stress = [(c,) for c in W.stress_counts(seed=3)]
@@ -727,6 +731,9 @@ def extras(headline_cases_block):
              note="1,024 fp32 tensors, log-uniform 256..65,536 elements (seed 3): pack with prescale 0.125, unpack; "
                   "200 repetitions timed; every kernel behind its predecessor on one stream")
     kernels("c2_fusion_stress", "c2")
+    pipeline("c2_fusion_stress_one_stream_completion_events", stress, F32, F32, 1.0, 0, 1.0, 1, 8, 200,
+             completion_events=True,
+             note="one stream, a pooled completion event behind every repetition")
     pipeline("c2_fusion_stress_two_streams", stress, F32, F32, 1.0, 0, 1.0, 2, 8, 200,
              note="consecutive repetitions alternate over two stream slots, each with its own fusion buffer; a pooled "
                   "completion event behind every repetition, as GPUOpContext::FinalizeGPUQueue records one per response")
