@@ -386,7 +386,7 @@ class PipelineRun:
     the same stream(s) and share the one fusion buffer of each stream slot."""
 
     def __init__(self, shapes, tdtype, bdtype, std, peers, fraction, streams, replicas, arrays=False,
-                 completion_events=None):
+                 completion_events=None, record_with_unpack=False):
         import torch
         from horovod_amd import dtype_size, workloads as W
         from horovod_amd.pipeline import AllreducePipeline
@@ -400,7 +400,8 @@ class PipelineRun:
             src = DeviceSet(self.counts, es, lambda n: randn_bytes(n, torch_dtype(tdtype), std, 1 + r))
             dst = DeviceSet(self.counts, es, zeros_bytes)
             pipe = AllreducePipeline(src.ptrs, dst.ptrs, self.counts, tdtype, bdtype, streams=shared, buffers=buffers,
-                                     array_entry_points=arrays, completion_events=completion_events)
+                                     array_entry_points=arrays, completion_events=completion_events,
+                                     record_with_unpack=record_with_unpack)
             buffers = pipe.buffers
             bs = dtype_size(pipe.buffer_dtype)
             # one buffer per peer, sized for the largest cycle's reduced chunk, serves every cycle
@@ -700,9 +701,9 @@ def extras(headline_cases_block):
     out = {}
 
     def pipeline(name, shapes, tdt, bdt, std, peers, fraction, streams, replicas, steps, arrays=False, note=None,
-                 completion_events=None):
+                 completion_events=None, record_with_unpack=False):
         run = PipelineRun(shapes, tdt, bdt, std, peers, fraction, streams, replicas, arrays=arrays,
-                          completion_events=completion_events)
+                          completion_events=completion_events, record_with_unpack=record_with_unpack)
         sec = timed(run.one_pass, run.sync, steps, max(2, steps // 10))
         out[name] = pipeline_figures(run, sec, streams, note)
         run.destroy()
@@ -724,6 +725,10 @@ def extras(headline_cases_block):
              completion_events=True,
              note="the headline pipeline with a pooled completion event recorded behind every cycle and waited for by "
                   "the host, as GPUOpContext::FinalizeGPUQueue does once per response (ops/gpu_operations.cc:50-98)")
+    pipeline("c1_resnet50_fp32_one_stream_completion_events_with_unpack", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0,
+             1, 4, 200, completion_events=True, record_with_unpack=True,
+             note="the same with the event bound to the unpack kernel's own completion (hvdhip_fusion_unpack_record) "
+                  "instead of recorded behind it")
 
     # C2: fusion stress, pack + unpack, 200 repetitions
     stress = [(c,) for c in W.stress_counts(seed=3)]
@@ -734,6 +739,9 @@ def extras(headline_cases_block):
     pipeline("c2_fusion_stress_one_stream_completion_events", stress, F32, F32, 1.0, 0, 1.0, 1, 8, 200,
              completion_events=True,
              note="one stream, a pooled completion event behind every repetition")
+    pipeline("c2_fusion_stress_one_stream_completion_events_with_unpack", stress, F32, F32, 1.0, 0, 1.0, 1, 8, 200,
+             completion_events=True, record_with_unpack=True,
+             note="one stream, the completion event of every repetition bound to its unpack kernel")
     pipeline("c2_fusion_stress_two_streams", stress, F32, F32, 1.0, 0, 1.0, 2, 8, 200,
              note="consecutive repetitions alternate over two stream slots, each with its own fusion buffer; a pooled "
                   "completion event behind every repetition, as GPUOpContext::FinalizeGPUQueue records one per response")

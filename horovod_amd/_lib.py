@@ -69,6 +69,7 @@ _PROTOTYPES = {
     "hvdhip_fusion_plan_num_chunks": (c_int64, [c_void_p]),
     "hvdhip_fusion_pack": (c_int, [c_void_p, c_void_p, c_double, c_uint, c_void_p]),
     "hvdhip_fusion_unpack": (c_int, [c_void_p, c_void_p, c_double, c_void_p]),
+    "hvdhip_fusion_unpack_record": (c_int, [c_void_p, c_void_p, c_double, c_void_p, c_void_p]),
     "hvdhip_reduce_sum": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "hvdhip_reduce_sum_k": (c_int, [c_void_p, _PV, c_int, c_int64, c_int, c_void_p]),
     "hvdhip_adasum_plan_create": (c_int, [POINTER(c_int), c_int, c_int, _PV]),

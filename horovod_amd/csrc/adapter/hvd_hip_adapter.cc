@@ -146,11 +146,24 @@ void GPUOpContext::InitGPUQueue(const std::vector<TensorTableEntry>& entries) {
   event_queue = std::queue<std::pair<std::string, Event>>();
   stream = &gpu_context_->streams[(size_t)global_state_->current_nccl_stream][entries[0].device];
   if (global_state_->timeline_initialized) gpu_context_->RecordEvent(event_queue, QUEUE, *stream);
+  completion_queued_ = false;
+}
+
+bool GPUOpContext::RecordsWithLastKernel() const {
+  return stream != nullptr && !global_state_->timeline_initialized && !global_state_->enable_async_completion;
+}
+
+void* GPUOpContext::QueueCompletionEvent() {
+  Event event = AcquireEvent(gpu_context_, *stream);
+  event_queue.emplace("", event);
+  completion_queued_ = true;
+  return *event.event;
 }
 
 void GPUOpContext::FinalizeGPUQueue(std::vector<TensorTableEntry>& entries,
                                     const std::function<void()>& error_check_callback) {
-  if (!global_state_->enable_async_completion) gpu_context_->RecordEvent(event_queue, "", *stream);
+  if (!global_state_->enable_async_completion && !completion_queued_)
+    gpu_context_->RecordEvent(event_queue, "", *stream);
   gpu_context_->SetDevice(entries[0].device);
   if (!global_state_->enable_async_completion || global_state_->timeline_initialized) {
     // with the timeline on, events are waited for on the host for accurate timings (ops/gpu_operations.cc:77-80)
@@ -261,7 +274,11 @@ void GPUAllreduce::ScaleMemcpyOutFusionBuffer(void* buffer_data, size_t buffer_l
                                               std::vector<TensorTableEntry>& entries) {
   if (global_state_->batch_d2d_memcopies) {
     hvdhip_fusion_plan* plan = PlanFor(entries);
-    int rc = hvdhip_fusion_unpack(plan, buffer_data, scale_factor, Stream(entries));
+    // The unpack is the response's last kernel: it takes the completion event along.
+    int rc = gpu_op_context_.RecordsWithLastKernel()
+                 ? hvdhip_fusion_unpack_record(plan, buffer_data, scale_factor, Stream(entries),
+                                               gpu_op_context_.QueueCompletionEvent())
+                 : hvdhip_fusion_unpack(plan, buffer_data, scale_factor, Stream(entries));
     if (rc == HVDHIP_ERR_UNSUPPORTED_DTYPE)
       throw std::logic_error("Type " + DataType_Name(entries[0].dtype) +
                              " not supported by BatchedScaledD2DMemcpyCudaImpl.");

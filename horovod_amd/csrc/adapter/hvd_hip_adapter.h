@@ -131,8 +131,16 @@ public:
                         const std::function<void()>& error_check_callback = nullptr);
   std::queue<std::pair<std::string, Event>> event_queue;
   gpuStream_t* stream = nullptr;
+  // Whether the response's last kernel should carry the completion event itself
+  // (hvdhip_fusion_unpack_record) instead of FinalizeGPUQueue recording one behind it: only when
+  // that event is the one thing FinalizeGPUQueue would record (no timeline, no asynchronous completion).
+  bool RecordsWithLastKernel() const;
+  // Takes an event from the pool, unrecorded, and queues it as the completion event ("" as in
+  // ops/gpu_operations.cc:82); the caller hands it to the launch that records it.
+  void* QueueCompletionEvent();
 
 private:
+  bool completion_queued_ = false;
   GPUContext* gpu_context_;
   GlobalState* global_state_;
 };

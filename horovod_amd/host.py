@@ -93,7 +93,12 @@ class FusionPlan:
         check(lib().hvdhip_fusion_pack(self.handle, buffer_ptr, float(scale), flags, stream.handle),
               "hvdhip_fusion_pack")
 
-    def unpack(self, buffer_ptr, scale, stream):
+    def unpack(self, buffer_ptr, scale, stream, event=None):
+        """event: a pooled event (ctypes.c_void_p) to be recorded behind the unpack as part of its launch."""
+        if event is not None:
+            check(lib().hvdhip_fusion_unpack_record(self.handle, buffer_ptr, float(scale), stream.handle, event),
+                  "hvdhip_fusion_unpack_record")
+            return
         check(lib().hvdhip_fusion_unpack(self.handle, buffer_ptr, float(scale), stream.handle),
               "hvdhip_fusion_unpack")
 

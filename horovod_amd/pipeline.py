@@ -44,7 +44,7 @@ class AllreducePipeline:
 
     def __init__(self, tensor_ptrs, output_ptrs, counts, tensor_dtype, buffer_dtype=None,
                  threshold=FUSION_THRESHOLD, num_streams=1, completion_events=None, streams=None,
-                 buffers=None, array_entry_points=False):
+                 buffers=None, array_entry_points=False, record_with_unpack=False):
         """completion_events: record a pooled event after every cycle and wait on those in
         synchronize(), as GPUOpContext::FinalizeGPUQueue does (about 2 us of stream time per
         event).  Default: on when cycles alternate over several streams, off for one stream,
@@ -59,7 +59,11 @@ class AllreducePipeline:
 
         array_entry_points: pack and unpack through hvdhip_batched_scaled_d2d_memcpy, the launcher
         that takes the copies as arrays with every call (ops/gpu_operations.cc:186-206), instead of
-        explicit plans; same-dtype buffers only."""
+        explicit plans; same-dtype buffers only.
+
+        record_with_unpack: a fused cycle's completion event goes out with its unpack
+        (hvdhip_fusion_unpack_record) instead of as a record of its own behind it."""
+        self.record_with_unpack = bool(record_with_unpack)
         self.tensor_dtype = int(tensor_dtype)
         self.buffer_dtype = int(tensor_dtype if buffer_dtype is None else buffer_dtype)
         ts, bs = dtype_size(self.tensor_dtype), dtype_size(self.buffer_dtype)
@@ -156,6 +160,12 @@ class AllreducePipeline:
             if cyc.plan is not None and self.array_entry_points:
                 in_buf, _, outs, sizes, n = cyc.arrays[slot]
                 self._copy_arrays(outs, in_buf, sizes, n, postscale, s)
+            elif cyc.plan is not None and self.completion_events and self.record_with_unpack:
+                ev = ctypes.c_void_p()
+                check(lib().hvdhip_event_acquire(s.handle, ctypes.byref(ev)), "hvdhip_event_acquire")
+                cyc.plan.unpack(self.buffers[slot].data_ptr(), postscale, s, event=ev)
+                self.pending.append((s, ev))
+                continue
             elif cyc.plan is not None:
                 cyc.plan.unpack(self.buffers[slot].data_ptr(), postscale, s)
             elif postscale != 1.0:

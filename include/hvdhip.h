@@ -264,6 +264,17 @@ int hvdhip_fusion_pack(hvdhip_fusion_plan* plan, void* fusion_buffer, double sca
 int hvdhip_fusion_unpack(hvdhip_fusion_plan* plan, const void* fusion_buffer,
                          double scale_factor, void* stream);
 
+/* hvdhip_fusion_unpack followed by hvdhip_event_record(event, stream), i.e. the
+ * unpack of a fused response and the completion event that
+ * GPUOpContext::FinalizeGPUQueue records behind it (ops/gpu_operations.cc:77-98,
+ * ops/cuda_operations.cc:88-100), as one submission: the event is bound to the
+ * unpack kernel's own completion signal instead of going onto the stream as a
+ * marker behind the kernel.  Query, synchronise and stream-wait see the event
+ * exactly as after the two separate calls.  A plan without payload records the
+ * event by itself.  Not for a stream that is being captured into a graph. */
+int hvdhip_fusion_unpack_record(hvdhip_fusion_plan* plan, const void* fusion_buffer,
+                                double scale_factor, void* stream, void* event);
+
 /* ------------------------------------------------------------------------ */
 /* Local reduce-sum: one GPU's share of a reduce-scatter                    */
 /* ------------------------------------------------------------------------ */

@@ -422,3 +422,87 @@ def test_rejected_arguments(gpu):
     with pytest.raises(horovod_amd.HvdHipError):
         plan.pack(t.data_ptr() + 8, 1.0, gpu.stream)  # fusion buffer must be 16-byte aligned
     plan.destroy()
+
+
+def _acquire(stream):
+    import ctypes
+    import horovod_amd
+    ev = ctypes.c_void_p()
+    horovod_amd.check(horovod_amd.lib().hvdhip_event_acquire(stream.handle, ctypes.byref(ev)), "hvdhip_event_acquire")
+    return ev
+
+
+def _event_done(ev):
+    import ctypes
+    import horovod_amd
+    done = ctypes.c_int(-1)
+    horovod_amd.check(horovod_amd.lib().hvdhip_event_query(ev, ctypes.byref(done)), "hvdhip_event_query")
+    return done.value
+
+
+@pytest.mark.parametrize("dtype,buffer_dtype,postscale", [(F32, F32, 1.0), (F32, F32, 0.5), (F16, F16, 0.25),
+                                                          (F32, F16, 1.0), (U8, U8, 1.0)])
+def test_unpack_that_records_its_completion_event(gpu, orc, dtype, buffer_dtype, postscale):
+    """hvdhip_fusion_unpack_record = unpack followed by a record of the event (ops/gpu_operations.cc:82):
+    once the event has completed the outputs are whole, for a host that waits on the event and
+    for another stream that waits on it; the pooled event serves again afterwards."""
+    import horovod_amd
+    import torch
+    L = horovod_amd.lib()
+    rng = np.random.default_rng(11)
+    es = SIZE_OF[dtype]
+    counts = [int(c) for c in rng.integers(1, 400000, 37)] + [3, 0, 1 << 21]
+    src, dst, offs, ooffs, vals = _build(gpu, rng, counts, dtype)
+    plan = gpu.H.FusionPlan([src.ptr(o) for o in offs], [dst.ptr(o) for o in ooffs], counts, dtype, buffer_dtype)
+    other = horovod_amd.Stream()
+    copy = torch.zeros_like(dst.dev)
+    try:
+        fb = gpu.empty(plan.buffer_len + 64)
+        cof = plan.offsets()
+        bes = SIZE_OF[buffer_dtype]
+        for turn, scale in enumerate((postscale, 1.0, postscale)):
+            plan.pack(fb.data_ptr(), 1.0, gpu.stream)
+            dst.dev.fill_(0x5A)
+            torch.cuda.synchronize()
+            ev = _acquire(gpu.stream)
+            plan.unpack(fb.data_ptr(), scale, gpu.stream, event=ev)
+            if turn == 1:
+                # a second stream waits for the event and copies the outputs; only that stream is waited for
+                horovod_amd.check(L.hvdhip_stream_wait_event(other.handle, ev), "hvdhip_stream_wait_event")
+                horovod_amd.check(L.hvdhip_memcpy_async(copy.data_ptr(), dst.dev.data_ptr(), dst.dev.numel(), 3,
+                                                        other.handle), "hvdhip_memcpy_async")
+                other.synchronize()
+                out = copy.cpu().numpy()
+            else:
+                horovod_amd.check(L.hvdhip_event_synchronize(ev), "hvdhip_event_synchronize")
+                out = dst.dev.cpu().numpy()  # no wait for the stream itself
+            assert _event_done(ev) == 1
+            horovod_amd.check(L.hvdhip_event_release(gpu.stream.handle, ev), "hvdhip_event_release")
+            buf = gpu.download(fb)
+            for i, c in enumerate(counts):
+                b = buf[cof[i]:cof[i] + c * bes]
+                if buffer_dtype != dtype:
+                    want = orc.scale_cast_f16_to_f32(b.view(np.uint16), scale)
+                elif scale == 1.0:
+                    want = b
+                else:
+                    want = orc.scale_buffer(b.view(NP_OF[dtype]) if dtype != F16 else b.view(np.uint16), scale, dtype)
+                got = out[ooffs[i]:ooffs[i] + c * es]
+                assert np.array_equal(got, want.view(np.uint8)), "turn %d tensor %d" % (turn, i)
+    finally:
+        gpu.sync()
+        other.destroy()
+        plan.destroy()
+
+
+def test_unpack_record_without_payload_records_the_event(gpu):
+    import horovod_amd
+    L = horovod_amd.lib()
+    plan = gpu.H.FusionPlan([], [], [], F32)
+    ev = _acquire(gpu.stream)
+    plan.unpack(0, 1.0, gpu.stream, event=ev)
+    horovod_amd.check(L.hvdhip_event_synchronize(ev), "hvdhip_event_synchronize")
+    assert _event_done(ev) == 1
+    horovod_amd.check(L.hvdhip_event_release(gpu.stream.handle, ev), "hvdhip_event_release")
+    assert L.hvdhip_fusion_unpack_record(plan.handle, None, 1.0, gpu.stream.handle, None) == -1  # event is NULL
+    plan.destroy()
