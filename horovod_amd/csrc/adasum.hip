@@ -231,8 +231,6 @@ struct Axpby {
     return (T)(pa + pb);
   }
 };
-// ScaledAddfp16, adasum.h:482-500: float coefficients, t = ca*a rounded to
-// fp32, r = fma(cb, b, t), rounded to half.
 // ScaledAddfp16, adasum.h:482-500: float coefficients, t = ca*a rounded to fp32, r = fma(cb, b, t)
 // rounded to fp32, then to half.  Both fp32 results are kept apart from what follows them: a fused
 // mixed-precision product would take a +0 addend and lose the sign of a -0 product, and a fused

@@ -69,7 +69,7 @@ constexpr int kMaxK = 8;  // peers per launch; more are folded in by further lau
 // A chunk of a few MiB (one GPU's share of a reduce-scatter) is a grid that the device holds all at
 // once, so whatever a workgroup does before its first load is paid in full by the launch.  The
 // arguments are therefore plain scalars in an order that lets the command processor hand the first
-// sixteen dwords over in registers (resident, n, tile, the tile order, the first four peers; a struct
+// fourteen dwords over in registers (resident, n, tile, the tile order, the first three peers; a struct
 // of pointers would not be preloaded), the rest arrives with one scalar load, and no branch stands
 // between a workgroup's start and its loads: with the prologue of three dependent scalar loads and
 // two branches that this replaces, the 7-peer sum of an 8 MiB chunk took 14.5 instead of 12.6 us.
