@@ -694,6 +694,54 @@ def allgather_extra(steps):
             "copies_per_step": len(counts) * (world + 1), "streams": 1, "replicas_rotated": len(sets)}
 
 
+def device_ceiling_extra(steps=20):
+    """What this device streams, measured in the same run: one 1 GiB buffer copied to another by the
+    library's copy kernel, by the runtime's own device-to-device hipMemcpyAsync, and by torch's copy
+    kernel, all on the same stream and timed with HIP events on it; three (source, destination) pairs
+    rotate.  The kernels above are to be read against these figures as well as against the nominal
+    8 TB/s."""
+    import torch
+    import horovod_amd
+    from horovod_amd import host as H
+    s = stream_pair()[0]
+    n = 1 << 30
+    pairs = [(randn_bytes(n, torch.float32, 1.0, 90 + i), torch.empty(n, dtype=torch.uint8, device="cuda"))
+             for i in range(3)]
+    torch.cuda.synchronize()
+    turn = [0]
+
+    def nxt():
+        turn[0] = (turn[0] + 1) % len(pairs)
+        return pairs[turn[0]]
+
+    def library():
+        src, dst = nxt()
+        H.batched_d2d_memcpy([dst.data_ptr()], [src.data_ptr()], [n], s)
+
+    memcpy = horovod_amd.lib().hvdhip_memcpy_async
+    D2D = 3  # HVDHIP_MEMCPY_D2D
+
+    def runtime():
+        src, dst = nxt()
+        horovod_amd.check(memcpy(dst.data_ptr(), src.data_ptr(), n, D2D, s.handle), "hvdhip_memcpy_async")
+
+    ext = torch.cuda.ExternalStream(s.handle.value)
+
+    def framework():
+        src, dst = nxt()
+        with torch.cuda.stream(ext):
+            dst.view(torch.float32).copy_(src.view(torch.float32))
+
+    out = {"bytes_copied": n, "algorithmic_bytes": 2 * n, "replicas_rotated": len(pairs)}
+    for name, fn in (("library_copy_kernel", library), ("hipMemcpyAsync_d2d", runtime), ("torch_copy_kernel", framework)):
+        sec = event_timed(fn, s, steps, 3)
+        out[name] = {"us": round(sec * 1e6, 1), "GB/s": round(2 * n / sec / 1e9, 1),
+                     "frac_of_8TBps": round(2 * n / sec / 1e9 / HBM_PEAK_GBS, 4)}
+    del pairs
+    torch.cuda.empty_cache()
+    return out
+
+
 def extras(headline_cases_block):
     import torch
     from horovod_amd import DTYPE, workloads as W
@@ -781,6 +829,7 @@ def extras(headline_cases_block):
                   "their tables resident in the library's cache after the first step")
 
     out["allgather_fusion_8ranks_pack_unpack"] = allgather_extra(200)
+    out["device_copy_1GiB_three_ways"] = device_ceiling_extra()
     return out
 
 
