@@ -100,6 +100,19 @@ def reduce_scatter_share(num_elements, world, fused=True):
     return num_elements // world
 
 
+def reduce_scatter_ranges(num_elements, world, fused=True):
+    """(first element, count) of what every local rank reduces, in rank order, as
+    NCCLHierarchicalAllreduce::Execute cuts a homogeneous job (ops/nccl_operations.cc:285-330): rank r
+    owns the share at r * share (buffer_data_at_rank_offset); the elements that do not divide
+    (single tensors only, a fused buffer is grown first) sit behind the last share and are reduced at
+    the last rank (root_rank = local_size - 1), whose range therefore runs to the end of the buffer."""
+    share = reduce_scatter_share(num_elements, world, fused)
+    if fused:
+        return [(r * share, share) for r in range(world)]
+    rest = num_elements % world
+    return [(r * share, share + (rest if r == world - 1 else 0)) for r in range(world)]
+
+
 def fuse(nbytes, threshold=FUSION_THRESHOLD, pad16=True):
     """Greedy fusion of a list of tensor byte sizes (one dtype, one set of scale
     factors) into groups of tensor indices, in the reference's queue discipline."""

@@ -24,6 +24,26 @@ def test_reduce_scatter_share_follows_the_reference():
     assert W.reduce_scatter_share(1003, 8, fused=False) == 125
 
 
+def test_reduce_scatter_ranges_cover_the_buffer_once():
+    # ops/nccl_operations.cc:308-330: shares at rank * share; the non-divisible rest of a single tensor
+    # goes to the last rank, right behind its share
+    for world in (1, 2, 3, 8):
+        for n in (0, 1, 7, 64, 1003, 65537):
+            for fused in (True, False):
+                ranges = W.reduce_scatter_ranges(n, world, fused)
+                assert len(ranges) == world
+                at = 0
+                for first, count in ranges:
+                    assert first == at and count >= 0
+                    at += count
+                if fused:
+                    assert at >= n and at % (world * 64) == 0 and at - n < world * 64
+                else:
+                    assert at == n
+                    assert all(c == n // world for _, c in ranges[:-1])
+    assert W.reduce_scatter_ranges(1003, 8, fused=False)[-1] == (875, 128)
+
+
 def test_bert_large_cycles_reduce_an_eighth():
     counts = [W.numel(s) for s in W.bert_large_shapes()]
     groups = W.fuse([2 * c for c in counts])
