@@ -7,6 +7,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <string>
+#include <tuple>
 #include <type_traits>
 #include <vector>
 
@@ -127,10 +128,19 @@ __device__ __forceinline__ uint32_t xcd_tile(uint32_t block, XcdOrder o) {
   return block < o.ordered ? permuted : block;
 }
 
-// Launches a streaming kernel: workgroups of kWG lanes, no dynamic LDS.
+// Launches a streaming kernel: workgroups of kWG lanes, no dynamic LDS.  The arguments are
+// converted to the kernel's own parameter types and handed to hipLaunchKernel by address; the
+// kernel is named by its host-side handle, never called through the pointer (a call through a
+// pointer depends on the compiler turning the handle into the launch stub at that call, which a
+// host build with -fsanitize=function does not do for a kernel that is not a template: its
+// launches vanish without an error).  The status is left for HVDHIP_CHECK_LAUNCH.
 template <typename... KArgs, typename... Args>
 inline void launch(void (*kernel)(KArgs...), uint32_t workgroups, hipStream_t stream, Args... args) {
-  hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(kWG), 0, stream, KArgs(args)...);
+  static_assert(sizeof...(KArgs) == sizeof...(Args), "one argument per kernel parameter");
+  std::tuple<KArgs...> values{KArgs(args)...};
+  void* addresses[sizeof...(KArgs) ? sizeof...(KArgs) : 1];
+  std::apply([&](auto&... v) { size_t i = 0; ((addresses[i++] = static_cast<void*>(&v)), ...); }, values);
+  (void)hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(workgroups), dim3(kWG), addresses, 0, stream);
 }
 
 // Store policy per kernel family (the three kinds of store are described in vecmem.h).  Lines
