@@ -18,3 +18,15 @@ def test_c_client_round_trip(gpu):
     assert r.returncode == 0, r.stdout + r.stderr
     assert "mismatches 0" in r.stdout
     print(r.stdout)
+
+
+def test_native_cache_stress(gpu):
+    """horovod_amd/csrc/examples/cache_stress.cc: copy-table cache with evictions on every call from
+    two threads, a stream destroyed under it, the cache at its default size, single-layer Adasum
+    plans beyond their capacity from two threads, plan and event lifetimes."""
+    exe = os.path.join(ROOT, "horovod_amd", "lib", "cache_stress")
+    assert os.path.exists(exe), "make -C horovod_amd/csrc"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "stress ok" in r.stdout
+    print(r.stdout)
