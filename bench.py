@@ -65,6 +65,9 @@ TRAFFIC_BYTES_MEASURED = {
     "c5.reduce_single": 475145691,
     "c5.scale_single": 318074457,
     "c5.unpack": 123480144,
+    "copy.library": 2155936353,
+    "copy.runtime": 2123025630,
+    "copy.torch": 2123026410,
 }
 TRAFFIC_PROFILE = {
     "c1": "profiles/c1_resnet50_fp32_kernels.txt",
@@ -72,9 +75,11 @@ TRAFFIC_PROFILE = {
     "c3": "profiles/c3_bert_large_fp16_kernels.txt",
     "c4": "profiles/c4_adasum_fp32_kernels.txt",
     "c5": "profiles/c5_gpt2_xl_fp16_kernels.txt",
+    "copy": "profiles/device_copy_1GiB_three_ways.txt",
 }
 
 CONFIGS = ("c1", "c2", "c3", "c4", "c5")
+KERNEL_ONLY = CONFIGS + ("c4h", "copy")
 
 
 def parse():
@@ -85,10 +90,11 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
-    ap.add_argument("--kernel-only", choices=CONFIGS + ("c4h",), default=None,
+    ap.add_argument("--kernel-only", choices=KERNEL_ONLY, default=None,
                     help="only the back-to-back kernel loops of one configuration (for rocprofv3 runs): c1 ResNet-50 "
                          "fp32 cycle, c2 fusion stress, c3 BERT-large fp32->fp16 cycle with 7 peers on the 1/8 share, "
-                         "c4 Adasum 2 x 2^25 fp32, c4h the same in fp16, c5 GPT-2 XL fp16 cycle and embedding; "
+                         "c4 Adasum 2 x 2^25 fp32, c4h the same in fp16, c5 GPT-2 XL fp16 cycle and embedding, copy 1 GiB moved by the "
+                         "library's kernel, by hipMemcpyAsync and by an elementwise kernel of torch; "
                          "--steps launches per kernel after --warmup")
     ap.add_argument("--calibrate", action="store_true",
                     help="only launch a plain 256 MiB device copy (scales rocprofv3 byte counters)")
@@ -349,6 +355,47 @@ def build_cases(cfg):
                      "Adasum combine of two vectors of 2^25 elements in 64 layers: first pass 2 N s bytes (leaves what "
                      "pays in the Infinity Cache), second pass 3 N s bytes; 4 pairs rotated", None, plan.destroy,
                      parts=[(k1, 2 * n * es), (k2, 3 * n * es)])]
+    if cfg == "copy":
+        # One GiB copied to another by the library's copy kernel, by the runtime's own device-to-device
+        # hipMemcpyAsync and by an elementwise kernel of torch: what this device streams, whoever asks.
+        import horovod_amd
+        n = 1 << 30
+        pairs = [(randn_bytes(n, torch.float32, 1.0, 90 + i), torch.empty(n, dtype=torch.uint8, device="cuda"))
+                 for i in range(3)]
+        torch.cuda.synchronize()
+        turn = [0]
+
+        def nxt():
+            turn[0] = (turn[0] + 1) % len(pairs)
+            return pairs[turn[0]]
+
+        def library():
+            src, dst = nxt()
+            H.batched_d2d_memcpy([dst.data_ptr()], [src.data_ptr()], [n], s)
+
+        memcpy = horovod_amd.lib().hvdhip_memcpy_async
+        D2D = 3  # HVDHIP_MEMCPY_D2D
+
+        def runtime():
+            src, dst = nxt()
+            horovod_amd.check(memcpy(dst.data_ptr(), src.data_ptr(), n, D2D, s.handle), "hvdhip_memcpy_async")
+
+        ext = torch.cuda.ExternalStream(s.handle.value)
+
+        def framework():
+            src, dst = nxt()
+            # an elementwise kernel of torch's own (Tensor.copy_ between buffers of one dtype is the
+            # runtime's hipMemcpyAsync again)
+            with torch.cuda.stream(ext):
+                torch.mul(src.view(torch.float32), 1.0, out=dst.view(torch.float32))
+
+        what = "1 GiB copied from one buffer to another; 3 (source, destination) pairs rotated"
+        return [Case("copy.library", "xfer_k<Copy<unsigned char>, 2, 0>", library, 2 * n,
+                     what + "; hvdhip_batched_d2d_memcpy with one entry", n // 4096),
+                Case("copy.runtime", "__amd_rocclr_copyBuffer", runtime, 2 * n,
+                     what + "; hipMemcpyAsync, device to device"),
+                Case("copy.torch", "at::native::vectorized_elementwise_kernel<4, MulFunctor<float>>", framework, 2 * n,
+                     what + "; torch.mul(x, 1.0, out=y) on fp32 views, on the same stream")]
     raise ValueError(cfg)
 
 
@@ -696,50 +743,16 @@ def allgather_extra(steps):
 
 def device_ceiling_extra(steps=20):
     """What this device streams, measured in the same run: one 1 GiB buffer copied to another by the
-    library's copy kernel, by the runtime's own device-to-device hipMemcpyAsync, and by torch's copy
-    kernel, all on the same stream and timed with HIP events on it; three (source, destination) pairs
-    rotate.  The kernels above are to be read against these figures as well as against the nominal
-    8 TB/s."""
+    library's copy kernel, by the runtime's own device-to-device hipMemcpyAsync, and by an elementwise
+    kernel of torch, all on the same stream and timed with HIP events on it (the `copy` kernel loops).  The
+    kernels above are to be read against these figures as well as against the nominal 8 TB/s."""
     import torch
-    import horovod_amd
-    from horovod_amd import host as H
-    s = stream_pair()[0]
-    n = 1 << 30
-    pairs = [(randn_bytes(n, torch.float32, 1.0, 90 + i), torch.empty(n, dtype=torch.uint8, device="cuda"))
-             for i in range(3)]
-    torch.cuda.synchronize()
-    turn = [0]
-
-    def nxt():
-        turn[0] = (turn[0] + 1) % len(pairs)
-        return pairs[turn[0]]
-
-    def library():
-        src, dst = nxt()
-        H.batched_d2d_memcpy([dst.data_ptr()], [src.data_ptr()], [n], s)
-
-    memcpy = horovod_amd.lib().hvdhip_memcpy_async
-    D2D = 3  # HVDHIP_MEMCPY_D2D
-
-    def runtime():
-        src, dst = nxt()
-        horovod_amd.check(memcpy(dst.data_ptr(), src.data_ptr(), n, D2D, s.handle), "hvdhip_memcpy_async")
-
-    ext = torch.cuda.ExternalStream(s.handle.value)
-
-    def framework():
-        src, dst = nxt()
-        with torch.cuda.stream(ext):
-            dst.view(torch.float32).copy_(src.view(torch.float32))
-
-    out = {"bytes_copied": n, "algorithmic_bytes": 2 * n, "replicas_rotated": len(pairs)}
-    for name, fn in (("library_copy_kernel", library), ("hipMemcpyAsync_d2d", runtime), ("torch_copy_kernel", framework)):
-        sec = event_timed(fn, s, steps, 3)
-        out[name] = {"us": round(sec * 1e6, 1), "GB/s": round(2 * n / sec / 1e9, 1),
-                     "frac_of_8TBps": round(2 * n / sec / 1e9 / HBM_PEAK_GBS, 4)}
-    del pairs
+    cases = build_cases("copy")
+    blocks = measure_cases(cases, steps=steps, warmup=3)
+    release(cases)
+    del cases
     torch.cuda.empty_cache()
-    return out
+    return {"kernels": blocks, "traffic_profile": TRAFFIC_PROFILE["copy"]}
 
 
 def extras(headline_cases_block):
