@@ -51,21 +51,21 @@ ROTATE = 6
 # named here under profiles/; tests/test_host_logic.py re-derives every figure from them.
 TRAFFIC_BYTES_MEASURED = {
     "c1.pack": 125571679,
-    "c1.reduce": 184760412,
-    "c1.unpack": 125581985,
-    "c2.pack": 93208344,
-    "c2.unpack": 92593204,
-    "c3.pack": 194434537,
-    "c3.reduce": 71756449,
-    "c3.unpack": 197803761,
-    "c4.combine": 662271124,
-    "c4h.combine": 331107195,
-    "c5.pack": 123465011,
-    "c5.reduce": 181653492,
-    "c5.reduce_single": 475145691,
-    "c5.scale_single": 318074457,
-    "c5.unpack": 123480144,
-    "copy.library": 2155936353,
+    "c1.reduce": 184760472,
+    "c1.unpack": 125579671,
+    "c2.pack": 93208463,
+    "c2.unpack": 92594017,
+    "c3.pack": 194421549,
+    "c3.reduce": 71756749,
+    "c3.unpack": 197818970,
+    "c4.combine": 662273259,
+    "c4h.combine": 331102123,
+    "c5.pack": 123465051,
+    "c5.reduce": 181653632,
+    "c5.reduce_single": 475145891,
+    "c5.scale_single": 318055645,
+    "c5.unpack": 123473213,
+    "copy.library": 2155922559,
     "copy.runtime": 2123025630,
     "copy.torch": 2123026410,
 }
@@ -232,8 +232,20 @@ def cycle_cases(cfg, counts, tdtype, bdtype, std, peers, share_world, stream, pa
     share = nelem if share_world == 1 else W.reduce_scatter_share(nelem, share_world)
     slack = 4096 * bs
     fb_pack = zeros_bytes(blen + slack)
-    fbs = [randn_bytes((blen + slack + 255) // 256 * 256, bt, std, seed0 + 50 + r) for r in range(ROTATE)]
-    peer_bufs = [[randn_bytes((share * bs + 255) // 256 * 256, bt, std, seed0 + 100 + 16 * r + p) for p in range(peers)]
+    # The rotating fusion buffers and peer chunks lie back to back (256-byte aligned) in one allocation,
+    # like the chunks of a staging buffer.  Buffers allocated one by one land wherever the driver finds
+    # physical pages, and the same kernel then measures 4 % apart from process to process (the ResNet-50
+    # reduce-sum: 29.5 or 30.8 us); and where they lie relative to each other matters to the memory
+    # controllers: the 7-peer sum of an 8 MiB share takes 12.3-12.4 us with its eight chunks back to back
+    # (8,135,424 bytes apart), 9 MiB or 8 MiB + 4 KiB apart, and 13.2-13.7 us with them exactly 8 or 16 MiB
+    # (or 8 MiB + 16 or 64 KiB) apart.
+    step = 256
+    fb_bytes = (blen + slack + step - 1) // step * step
+    peer_bytes = (share * bs + step - 1) // step * step
+    arena = randn_bytes(ROTATE * (fb_bytes + peers * peer_bytes), bt, std, seed0 + 50)
+    fbs = [arena[r * fb_bytes:(r + 1) * fb_bytes] for r in range(ROTATE)]
+    at = ROTATE * fb_bytes
+    peer_bufs = [[arena[at + (r * peers + p) * peer_bytes:at + (r * peers + p + 1) * peer_bytes] for p in range(peers)]
                  for r in range(ROTATE)]
     torch.cuda.synchronize()
     payload = sum(counts)
@@ -545,9 +557,9 @@ def cpu_baseline_resnet(budget_s=12.0):
 
 
 def cpu_extras(budget_s=2.5):
-    """The CPU oracle on one core over bounded samples of the other configurations, in the same
-    algorithmic bytes as the GPU figures: the stress set, one 42-tensor BERT-large cycle (cast and
-    scale fused into the copy, which flatters the CPU), the whole Adasum pair, one GPT-2 XL layer."""
+    """The CPU oracle on one core over the other configurations, whole sets, in the same algorithmic
+    bytes as the GPU figures: the stress set, BERT-large in its 11 cycles (cast and scale fused into
+    the copy, which flatters the CPU), the Adasum pair, GPT-2 XL in its 49 cycles."""
     from ctypes import c_double, c_int, c_int64, c_void_p
     from horovod_amd import workloads as W
     ou, L = _oracle()
@@ -560,6 +572,12 @@ def cpu_extras(budget_s=2.5):
 
     def ptrs(arrays):
         return (c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
+
+    def rep(block, c):
+        """c values: the block, repeated as often as it takes."""
+        if c <= block.size:
+            return block[:c].copy()
+        return np.concatenate([block] * (c // block.size) + [block[:c % block.size]])
 
     def run(name, fn, nbytes, sample):
         fn()
@@ -588,28 +606,35 @@ def cpu_extras(budget_s=2.5):
 
     run("c2_fusion_stress", stress, 4 * 4 * n, "the whole 1,024-tensor set")
 
-    # BERT-large, one cycle of 42 tensors: fp32 -> fp16 with prescale, 7 peers on 1/8, fp16 -> fp32
-    counts = [W.numel(s) for s in W.bert_large_shapes()][7:49]
-    ts = [(rng.standard_normal(c, dtype=np.float32) * np.float32(1e-4)) for c in counts]
+    # BERT-large, the whole set in its 11 cycles: fp32 -> fp16 with prescale, 7 peers on 1/8, fp16 -> fp32
+    counts = [W.numel(s) for s in W.bert_large_shapes()]
+    groups = W.fuse([2 * c for c in counts])
+    # (the tensors repeat one block of random values: the CPU's time does not depend on the values,
+    # and drawing 336 M of them would take longer than the measurement)
+    block = rng.standard_normal(1 << 24, dtype=np.float32) * np.float32(1e-4)
+    ts = [rep(block, c) for c in counts]
     outs = [np.empty_like(t) for t in ts]
-    n = sum(counts)
-    hbuf = np.zeros(n + 4096, np.uint16)
-    share = W.reduce_scatter_share(n, 8)
-    peers = [rng.integers(0, 0x0400, share, dtype=np.uint16) for _ in range(7)]
+    sizes = [sum(counts[i] for i in g) for g in groups]
+    shares = [W.reduce_scatter_share(n, 8) for n in sizes]
+    hbuf = np.zeros(max(sizes) + 4096, np.uint16)
+    peers = [[rng.integers(0, 0x0400, sh, dtype=np.uint16) for _ in range(7)] for sh in shares]
 
     def bert():
-        off = 0
-        for t, c in zip(ts, counts):
-            L.orc_scale_cast_f32_to_f16_f16c(P(t), P(hbuf, 2 * off), c_int64(c), c_double(0.125))
-            off += c
-        for p in peers:
-            L.orc_float16_sum(P(p), P(hbuf), c_int64(share))
-        off = 0
-        for o, c in zip(outs, counts):
-            L.orc_scale_cast_f16_to_f32_f16c(P(hbuf, 2 * off), P(o), c_int64(c), c_double(1.0))
-            off += c
+        for g, share, ps in zip(groups, shares, peers):
+            off = 0
+            for i in g:
+                L.orc_scale_cast_f32_to_f16_f16c(P(ts[i]), P(hbuf, 2 * off), c_int64(counts[i]), c_double(0.125))
+                off += counts[i]
+            for p in ps:
+                L.orc_float16_sum(P(p), P(hbuf), c_int64(share))
+            off = 0
+            for i in g:
+                L.orc_scale_cast_f16_to_f32_f16c(P(hbuf, 2 * off), P(outs[i]), c_int64(counts[i]), c_double(1.0))
+                off += counts[i]
 
-    run("c3_bert_large_fp32_to_fp16_7peers_eighth_share", bert, 6 * n + 9 * 2 * share + 6 * n, "one 42-tensor cycle")
+    run("c3_bert_large_fp32_to_fp16_7peers_eighth_share", bert,
+        sum(12 * n + 9 * 2 * sh for n, sh in zip(sizes, shares)), "the whole 397-tensor set in %d cycles" % len(groups))
+    del ts, outs, peers, block
 
     # Adasum: the whole pair, in place on a (values stay finite from repetition to repetition)
     n = 1 << 25
@@ -621,23 +646,34 @@ def cpu_extras(budget_s=2.5):
         lambda: L.orc_adasum_pairwise(P(a), P(b), c_int(F32), P(lc), c_int(64), P(nd), P(co)), 5 * n * 4,
         "the whole pair")
 
-    # GPT-2 XL: one transformer layer (12 fp16 tensors, 61.5 MB)
-    counts = [W.numel(s) for s in W.gpt2_xl_shapes()][2:14]
-    ts = [rng.integers(0, 0x3c00, c, dtype=np.uint16) for c in counts]
+    # GPT-2 XL, the whole set: 48 fused cycles (memcpy pack, ScaleBuffer in place, sum with the peer buffer,
+    # memcpy unpack: 7P) and the embedding by itself (scale from tensor to output, sum in place: 5P)
+    counts = [W.numel(s) for s in W.gpt2_xl_shapes()]
+    groups = W.fuse([2 * c for c in counts])
+    block = rng.integers(0x0400, 0x3c00, 1 << 25, dtype=np.uint16)  # normal halves below 1, repeated
+    ts = [rep(block, c) for c in counts]
     outs = [np.empty_like(t) for t in ts]
-    n, k = sum(counts), len(counts)
-    nb = np.array([2 * c for c in counts], np.int64)
-    hbuf = np.zeros(n, np.uint16)
-    peer = rng.integers(0, 0x3c00, n, dtype=np.uint16)
-    tp2, op2 = ptrs(ts), ptrs(outs)
+    sizes = [sum(counts[i] for i in g) for g in groups]
+    peers = [rep(block[12345:], n) for n in sizes]
+    hbuf = np.zeros(max(n for n, g in zip(sizes, groups) if len(g) > 1), np.uint16)
+    args = []
+    for g, n in zip(groups, sizes):
+        nb = np.array([2 * counts[i] for i in g], np.int64)
+        args.append((ptrs([ts[i] for i in g]), ptrs([outs[i] for i in g]), nb, len(g), n))
 
     def gpt2():
-        L.orc_pack(tp2, P(nb), c_int(k), P(hbuf))
-        L.orc_scale_buffer(P(hbuf), P(hbuf), c_int64(n), c_double(0.125), c_int(F16))
-        L.orc_float16_sum(P(peer), P(hbuf), c_int64(n))
-        L.orc_unpack(P(hbuf), op2, P(nb), c_int(k))
+        for (tp2, op2, nb, k, n), g, peer in zip(args, groups, peers):
+            if k == 1:
+                L.orc_scale_buffer(P(ts[g[0]]), P(outs[g[0]]), c_int64(n), c_double(0.125), c_int(F16))
+                L.orc_float16_sum(P(peer), P(outs[g[0]]), c_int64(n))
+                continue
+            L.orc_pack(tp2, P(nb), c_int(k), P(hbuf))
+            L.orc_scale_buffer(P(hbuf), P(hbuf), c_int64(n), c_double(0.125), c_int(F16))
+            L.orc_float16_sum(P(peer), P(hbuf), c_int64(n))
+            L.orc_unpack(P(hbuf), op2, P(nb), c_int(k))
 
-    run("c5_gpt2_xl_fp16_two_streams", gpt2, 7 * 2 * n, "one transformer layer (12 tensors)")
+    run("c5_gpt2_xl_fp16_two_streams", gpt2, sum((7 if len(g) > 1 else 5) * 2 * n for g, n in zip(groups, sizes)),
+        "the whole 580-tensor set in %d cycles" % len(groups))
     return out
 
 
