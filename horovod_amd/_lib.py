@@ -43,6 +43,7 @@ _PROTOTYPES = {
     "hvdhip_set_device": (c_int, [c_int]),
     "hvdhip_stream_create": (c_int, [_PV]),
     "hvdhip_stream_destroy": (c_int, [c_void_p]),
+    "hvdhip_stream_forget": (c_int, [c_void_p]),
     "hvdhip_stream_synchronize": (c_int, [c_void_p]),
     "hvdhip_stream_wait_event": (c_int, [c_void_p, c_void_p]),
     "hvdhip_event_acquire": (c_int, [c_void_p, _PV]),

@@ -17,6 +17,6 @@ def build(force=False, jobs=8):
 
 def ensure_built():
     """Builds the libraries only if one of them is missing; never replaces an existing build."""
-    need = [os.path.join(_HERE, "lib", n) for n in ("libhvdhip.so", "libhvdhip_adapter.so", "c_client", "cache_stress")]
+    need = [os.path.join(_HERE, "lib", n) for n in ("libhvdhip.so", "libhvdhip_tuning.so", "libhvdhip_adapter.so", "c_client", "cache_stress")]
     if not all(os.path.exists(p) for p in need):
         build()

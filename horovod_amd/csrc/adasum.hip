@@ -428,21 +428,18 @@ constexpr uint64_t kKeepBothBytes = (uint64_t)160 << 20;  // largest pair (both 
 inline int keep_mode(uint64_t vector_bytes) { return 2 * vector_bytes <= kKeepBothBytes ? 2 : 1; }
 
 template <int KEEP>
-void launch_dot_partials(hvdhip_adasum_plan* p, const void* a, const void* b, hipStream_t s) {
+hipError_t launch_dot_partials(hvdhip_adasum_plan* p, const void* a, const void* b, hipStream_t s) {
   const DevTables& t = p->tables;
   switch (p->dtype) {
   case HVDHIP_FLOAT16:
-    launch(dot_partials_k<half_t, KEEP>, t.nchunks, s, t.chunks, static_cast<const half_t*>(a),
-           static_cast<const half_t*>(b), p->partials);
-    break;
+    return launch(dot_partials_k<half_t, KEEP>, t.nchunks, s, t.chunks, static_cast<const half_t*>(a),
+                  static_cast<const half_t*>(b), p->partials);
   case HVDHIP_FLOAT32:
-    launch(dot_partials_k<float, KEEP>, t.nchunks, s, t.chunks, static_cast<const float*>(a),
-           static_cast<const float*>(b), p->partials);
-    break;
+    return launch(dot_partials_k<float, KEEP>, t.nchunks, s, t.chunks, static_cast<const float*>(a),
+                  static_cast<const float*>(b), p->partials);
   default:
-    launch(dot_partials_k<double, KEEP>, t.nchunks, s, t.chunks, static_cast<const double*>(a),
-           static_cast<const double*>(b), p->partials);
-    break;
+    return launch(dot_partials_k<double, KEEP>, t.nchunks, s, t.chunks, static_cast<const double*>(a),
+                  static_cast<const double*>(b), p->partials);
   }
 }
 
@@ -452,27 +449,23 @@ int plan_dot_norms(hvdhip_adasum_plan* p, const void* a, const void* b, hipStrea
   if (p->nlayers == 0) return 0;
   const DevTables& t = p->tables;
   if (t.nchunks > 0) {
-    if (keep_mode((uint64_t)p->total * (uint64_t)dtype_size(p->dtype)) == 2)
-      launch_dot_partials<2>(p, a, b, s);
-    else
-      launch_dot_partials<1>(p, a, b, s);
-    HVDHIP_CHECK_LAUNCH("dot_partials_k");
+    const bool both = keep_mode((uint64_t)p->total * (uint64_t)dtype_size(p->dtype)) == 2;
+    HVDHIP_CHECK_LAUNCH("dot_partials_k", both ? launch_dot_partials<2>(p, a, b, s) : launch_dot_partials<1>(p, a, b, s));
   }
   if (!finalize) return 0;
-  launch(finalize_k, (uint32_t)p->nlayers, s, p->layers, p->partials,
-                     p->normdots, p->coeffs, std::sqrt(DBL_MIN));
-  HVDHIP_CHECK_LAUNCH("finalize_k");
+  HVDHIP_CHECK_LAUNCH("finalize_k", launch(finalize_k, (uint32_t)p->nlayers, s, p->layers, p->partials, p->normdots,
+                                           p->coeffs, std::sqrt(DBL_MIN)));
   return 0;
 }
 
 template <typename T, bool FUSED>
-void launch_scaled_add(hvdhip_adasum_plan* p, void* a, const void* b, const double* coeffs,
-                       double ca, double cb, hipStream_t s) {
+hipError_t launch_scaled_add(hvdhip_adasum_plan* p, void* a, const void* b, const double* coeffs,
+                             double ca, double cb, hipStream_t s) {
   const DevTables& t = p->tables;
-  with_store_policy(Stores::kAdasum, [&](auto st) {
-    launch(scaled_add_k<T, FUSED, decltype(st)::value>, t.nchunks, s, t.chunks, static_cast<T*>(a),
-           static_cast<const T*>(b), coeffs, ca, cb, p->layers, p->partials, p->normdots, p->coeffs,
-           std::sqrt(DBL_MIN), (uint32_t)p->nlayers);
+  return with_store_policy(Stores::kAdasum, [&](auto st) {
+    return launch(scaled_add_k<T, FUSED, decltype(st)::value>, t.nchunks, s, t.chunks, static_cast<T*>(a),
+                  static_cast<const T*>(b), coeffs, ca, cb, p->layers, p->partials, p->normdots, p->coeffs,
+                  std::sqrt(DBL_MIN), (uint32_t)p->nlayers);
   });
 }
 
@@ -480,12 +473,13 @@ template <bool FUSED>
 int scaled_add_by_dtype(hvdhip_adasum_plan* p, void* a, const void* b, const double* coeffs,
                         double ca, double cb, hipStream_t s) {
   if (p->tables.nchunks == 0) return 0;
+  hipError_t status;
   switch (p->dtype) {
-  case HVDHIP_FLOAT16: launch_scaled_add<half_t, FUSED>(p, a, b, coeffs, ca, cb, s); break;
-  case HVDHIP_FLOAT32: launch_scaled_add<float, FUSED>(p, a, b, coeffs, ca, cb, s); break;
-  default: launch_scaled_add<double, FUSED>(p, a, b, coeffs, ca, cb, s); break;
+  case HVDHIP_FLOAT16: status = launch_scaled_add<half_t, FUSED>(p, a, b, coeffs, ca, cb, s); break;
+  case HVDHIP_FLOAT32: status = launch_scaled_add<float, FUSED>(p, a, b, coeffs, ca, cb, s); break;
+  default: status = launch_scaled_add<double, FUSED>(p, a, b, coeffs, ca, cb, s); break;
   }
-  HVDHIP_CHECK_LAUNCH("scaled_add_k");
+  HVDHIP_CHECK_LAUNCH("scaled_add_k", status);
   return 0;
 }
 
@@ -583,6 +577,25 @@ void unpin(OneLayerEntry* e) {
 }
 
 }  // namespace
+
+// The stream is idle and about to be destroyed: the plans made for it would never be found again
+// (a later stream at the same address on another device aside) and hold device memory.
+void hvdhip::adasum_forget_stream(hipStream_t stream) {
+  OneLayerCache& c = one_layer_cache();
+  std::vector<hvdhip_adasum_plan*> dead;
+  {
+    std::lock_guard<std::mutex> g(c.mu);
+    for (auto it = c.lru.begin(); it != c.lru.end();) {
+      if (it->stream == stream && it->users == 0) {
+        dead.push_back(it->plan);
+        it = c.lru.erase(it);
+      } else {
+        ++it;
+      }
+    }
+  }
+  for (hvdhip_adasum_plan* p : dead) (void)hvdhip_adasum_plan_destroy(p);  // waits for the device: outside the mutex
+}
 
 extern "C" {
 
@@ -820,9 +833,9 @@ int hvdhip_adasum_combine_static(void* a, const void* b, int dtype, int count, d
   // The array keeps what the last call left: the tables are rewritten for this count, and every
   // partial sum that is read is written first by this call's first pass.
   const uint32_t run = xcd_run(nchunks, chunk_bytes(Family::kAdasum), true);
-  launch(one_layer_tables_k, (uint32_t)(nchunks / kWG + 1), s, view.tables.chunks, view.layers,
-         (uint32_t)nchunks, (uint64_t)count, chunk_units, run);
-  HVDHIP_CHECK_LAUNCH("one_layer_tables_k");
+  HVDHIP_CHECK_LAUNCH("one_layer_tables_k",
+                      launch(one_layer_tables_k, (uint32_t)(nchunks / kWG + 1), s, view.tables.chunks, view.layers,
+                             (uint32_t)nchunks, (uint64_t)count, chunk_units, run));
   const bool fused = fused_coeffs(&view);
   rc = plan_dot_norms(&view, a, b, s, !fused);
   if (rc) return rc;

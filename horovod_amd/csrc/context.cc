@@ -69,6 +69,9 @@ int ok() {
 }
 
 uint32_t chunk_bytes(Family f) {
+#ifdef HVDHIP_TUNING
+  // Tuning builds only (libhvdhip_tuning.so): HVDHIP_CHUNK_BYTES, a multiple of 4096, replaces every
+  // family's chunk size, so that tests reach the kernels' multi-vector loops.
   static uint32_t forced = [] {
     const char* e = getenv("HVDHIP_CHUNK_BYTES");
     if (e) {
@@ -78,6 +81,7 @@ uint32_t chunk_bytes(Family f) {
     return 0u;
   }();
   if (forced) return forced;
+#endif
   switch (f) {
   case Family::kXfer: return kXferChunkBytes;
   case Family::kXferNarrowing: return kXferNarrowingChunkBytes;
@@ -128,10 +132,15 @@ uint32_t xcd_run(uint64_t nchunks, uint32_t chunk_bytes, bool long_runs) {
 int store_policy(Stores family) {
   constexpr unsigned kDefaultThrough = 1u << (unsigned)Stores::kPack | 1u << (unsigned)Stores::kPackNarrowing |
                                        1u << (unsigned)Stores::kReduceFew | 1u << (unsigned)Stores::kReduceMany;
+#ifdef HVDHIP_TUNING
+  // Tuning builds only: HVDHIP_WRITE_THROUGH=<mask> (bit = enumerator value) replaces the table.
   static const unsigned through = [] {
     const char* e = std::getenv("HVDHIP_WRITE_THROUGH");
     return e ? (unsigned)std::strtoul(e, nullptr, 0) : kDefaultThrough;
   }();
+#else
+  constexpr unsigned through = kDefaultThrough;
+#endif
   return (through >> (unsigned)family) & 1u;
 }
 
@@ -241,12 +250,16 @@ int hvdhip_stream_create(void** stream) {
   return ok();
 }
 
-int hvdhip_stream_destroy(void* stream) {
-  hipStream_t s = static_cast<hipStream_t>(stream);
+namespace {
+// Waits for the stream and drops everything the library keeps per stream: idle pooled events,
+// the streams' marks on cached copy tables, single-layer Adasum plans.
+int forget_stream(hipStream_t s) {
   int dev = 0;
   HVDHIP_CHECK(hipGetDevice(&dev));
+  // Work still queued completes first, so that nothing the library remembers about the stream
+  // (tables a launch on it reads) outlives it.
+  HVDHIP_CHECK(hipStreamSynchronize(s));
   {
-    // Drop the stream's idle events with it.
     EventPools& p = pools();
     std::lock_guard<std::mutex> g(p.mu);
     auto key = std::make_pair(dev, s);
@@ -257,12 +270,23 @@ int hvdhip_stream_destroy(void* stream) {
     }
     p.filled.erase(key);
   }
-  // Work still queued completes first, so that nothing the library remembers about the stream
-  // (tables a launch on it reads) outlives it.
-  HVDHIP_CHECK(hipStreamSynchronize(s));
   copy_cache_forget_stream(s);
+  adasum_forget_stream(s);
+  return 0;
+}
+}  // namespace
+
+int hvdhip_stream_destroy(void* stream) {
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int rc = forget_stream(s);
+  if (rc) return rc;
   HVDHIP_CHECK(hipStreamDestroy(s));
   return ok();
+}
+
+int hvdhip_stream_forget(void* stream) {
+  int rc = forget_stream(static_cast<hipStream_t>(stream));
+  return rc ? rc : ok();
 }
 
 int hvdhip_stream_synchronize(void* stream) {

@@ -3,6 +3,7 @@
 #define HVDHIP_INTERNAL_H
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstdint>
 #include <cstdio>
@@ -32,10 +33,11 @@ int ok();
     }                                                                               \
   } while (0)
 
-// Checks the launch that has just been issued.
-#define HVDHIP_CHECK_LAUNCH(name)                                                   \
+// Checks the status that launch() returned for the kernel `name`.  Only that value is looked at:
+// the thread's last-error state belongs to the application and is neither read nor cleared.
+#define HVDHIP_CHECK_LAUNCH(name, status)                                           \
   do {                                                                              \
-    hipError_t hvdhip_e_ = hipGetLastError();                                       \
+    hipError_t hvdhip_e_ = (status);                                                \
     if (hvdhip_e_ != hipSuccess)                                                    \
       return ::hvdhip::fail((int)hvdhip_e_, "%s launch failed: %s", name,           \
                             hipGetErrorString(hvdhip_e_));                          \
@@ -55,11 +57,9 @@ inline int64_t dtype_size(int dtype) {
 // (float)scale, or that value rounded to half (nearest even) and widened again.
 float fp16_scale_factor(double scale);
 
-// Threads per workgroup of every streaming kernel: four wave64 wavefronts.
-#ifndef HVDHIP_WG
-#define HVDHIP_WG 256
-#endif
-constexpr int kWG = HVDHIP_WG;
+// Threads per workgroup of every streaming kernel: four wave64 wavefronts.  (Workgroups of 64, 128,
+// 512 and 1,024 lanes measured 0-9 % slower.)
+constexpr int kWG = 256;
 static_assert(kWG % 64 == 0 && kWG >= 64 && kWG <= 1024, "whole wave64 wavefronts");
 
 // A launch may not exceed 2^32 - 1 threads in x.  Contiguous kernels cover larger buffers
@@ -72,7 +72,8 @@ constexpr uint64_t kMaxWorkgroups = 1ull << 23;
 // the HBM peak, against about 70 % for 16-32 KiB per workgroup; the occupancy
 // of many small workgroups hides latency better than unrolling inside one.
 // The Adasum reduction pays a workgroup-wide tree per chunk and prefers 16 KiB.
-// HVDHIP_CHUNK_BYTES (a multiple of 4096) overrides all three, for tuning.
+// (A build with -DHVDHIP_TUNING reads HVDHIP_CHUNK_BYTES to override all of them; the shipped
+// library reads nothing.)
 enum class Family { kXfer, kXferNarrowing, kReduce, kAdasum };
 constexpr uint32_t kXferChunkBytes = 4096;
 constexpr uint32_t kXferNarrowingChunkBytes = 8192;  // fp32 -> fp16 pack: 32 bytes in, 16 out per lane
@@ -129,18 +130,27 @@ __device__ __forceinline__ uint32_t xcd_tile(uint32_t block, XcdOrder o) {
 }
 
 // Launches a streaming kernel: workgroups of kWG lanes, no dynamic LDS.  The arguments are
-// converted to the kernel's own parameter types and handed to hipLaunchKernel by address; the
-// kernel is named by its host-side handle, never called through the pointer (a call through a
-// pointer depends on the compiler turning the handle into the launch stub at that call, which a
-// host build with -fsanitize=function does not do for a kernel that is not a template: its
-// launches vanish without an error).  The status is left for HVDHIP_CHECK_LAUNCH.
+// converted to the kernel's own parameter types and handed over by address; the kernel is named
+// by its host-side handle, never called through the pointer (a call through a pointer depends on
+// the compiler turning the handle into the launch stub at that call, which a host build with
+// -fsanitize=function does not do for a kernel that is not a template: its launches vanish
+// without an error).  Returns the launch call's own status, for HVDHIP_CHECK_LAUNCH.
+// completion: an event to be bound to the kernel's completion signal (the launch's stop event).
 template <typename... KArgs, typename... Args>
-inline void launch(void (*kernel)(KArgs...), uint32_t workgroups, hipStream_t stream, Args... args) {
+inline hipError_t launch_with(hipEvent_t completion, void (*kernel)(KArgs...), uint32_t workgroups,
+                              hipStream_t stream, Args... args) {
   static_assert(sizeof...(KArgs) == sizeof...(Args), "one argument per kernel parameter");
   std::tuple<KArgs...> values{KArgs(args)...};
   void* addresses[sizeof...(KArgs) ? sizeof...(KArgs) : 1];
   std::apply([&](auto&... v) { size_t i = 0; ((addresses[i++] = static_cast<void*>(&v)), ...); }, values);
-  (void)hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(workgroups), dim3(kWG), addresses, 0, stream);
+  const void* handle = reinterpret_cast<const void*>(kernel);
+  if (completion)
+    return hipExtLaunchKernel(handle, dim3(workgroups), dim3(kWG), addresses, 0, stream, nullptr, completion, 0);
+  return hipLaunchKernel(handle, dim3(workgroups), dim3(kWG), addresses, 0, stream);
+}
+template <typename... KArgs, typename... Args>
+inline hipError_t launch(void (*kernel)(KArgs...), uint32_t workgroups, hipStream_t stream, Args... args) {
+  return launch_with(nullptr, kernel, workgroups, stream, args...);
 }
 
 // Store policy per kernel family (the three kinds of store are described in vecmem.h).  Lines
@@ -151,7 +161,8 @@ inline void launch(void (*kernel)(KArgs...), uint32_t workgroups, hipStream_t st
 // instead of 16.3 us) and saves the reader more (the unpack behind it: 12 instead of 16.4 us), so the
 // kernels whose output the next kernel reads write through, and the ones whose output leaves the
 // pipeline (unpack, batched copies, Adasum's scaled add, a whole-buffer scale) do not.
-// HVDHIP_WRITE_THROUGH=<mask> (bit = enumerator value) overrides the built-in table, for tuning.
+// (A build with -DHVDHIP_TUNING reads HVDHIP_WRITE_THROUGH=<mask>, bit = enumerator value, to
+// override the built-in table; the shipped library reads nothing.)
 enum class Stores {
   kPack = 0,        // same-width pack into the fusion buffer
   kUnpack = 1,      // same-width unpack out of it
@@ -165,13 +176,11 @@ enum class Stores {
 };
 int store_policy(Stores family);  // a StorePolicy value
 
-// Calls f(std::integral_constant<int, policy>) for the family's policy.
+// Calls f(std::integral_constant<int, policy>) for the family's policy and returns what it returns.
 template <typename F>
-inline void with_store_policy(Stores family, F&& f) {
-  if (store_policy(family))
-    f(std::integral_constant<int, 1>());
-  else
-    f(std::integral_constant<int, 0>());
+inline auto with_store_policy(Stores family, F&& f) {
+  if (store_policy(family)) return f(std::integral_constant<int, 1>());
+  return f(std::integral_constant<int, 0>());
 }
 
 // One contiguous run of elements to transfer (host side only).  `tensor` and
@@ -236,6 +245,8 @@ class DeviceGuard {
 
 // Tells the copy-table caches that `stream` has been synchronised and is about to be destroyed.
 void copy_cache_forget_stream(hipStream_t stream);
+// Destroys the single-layer Adasum plans kept for `stream` (idle, about to be destroyed).
+void adasum_forget_stream(hipStream_t stream);
 
 // Uploads a ready-made chunk table.
 int upload_chunks(const std::vector<Chunk>& chunks, DevTables* out);

@@ -133,11 +133,11 @@ int launch_k(void* resident, const void* const* incoming, int64_t n, hipStream_t
     const T* p[kMaxK];
     for (int k = 0; k < kMaxK; ++k) p[k] = k < K ? static_cast<const T*>(incoming[k]) + done : nullptr;
     const XcdOrder order = xcd_order(blocks, tile * (uint32_t)sizeof(T));
-    with_store_policy(K <= 2 ? Stores::kReduceFew : Stores::kReduceMany, [&](auto st) {
-      launch(reduce_k<T, K, decltype(st)::value>, blocks, stream, static_cast<T*>(resident) + done, slice, tile,
-             order.shift, order.ordered, 0u, p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
+    const hipError_t status = with_store_policy(K <= 2 ? Stores::kReduceFew : Stores::kReduceMany, [&](auto st) {
+      return launch(reduce_k<T, K, decltype(st)::value>, blocks, stream, static_cast<T*>(resident) + done, slice,
+                    tile, order.shift, order.ordered, 0u, p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
     });
-    HVDHIP_CHECK_LAUNCH("reduce_k");
+    HVDHIP_CHECK_LAUNCH("reduce_k", status);
     done += slice;
     left -= slice;
   }

@@ -61,10 +61,7 @@ struct Arr {
 };
 
 // Streaming data is touched once: the non-temporal hint keeps it from
-// displacing useful lines in L2 and the Infinity Cache.
-#ifndef HVDHIP_NONTEMPORAL
-#define HVDHIP_NONTEMPORAL 1
-#endif
+// displacing useful lines in L2 and the Infinity Cache (+5-15 % measured against plain accesses).
 
 // NT = false loads without the hint, for data that a later kernel reads again while it can
 // still be in the Infinity Cache.
@@ -79,7 +76,7 @@ __device__ __forceinline__ Arr<T, N> ldv(gptr<const T> p) {
   } else {
   typedef typename Raw<(int)sizeof(T) * N, (int)alignof(T)>::type R;
   typename RawSel<(int)sizeof(T) * N>::type r;
-  if constexpr (NT && HVDHIP_NONTEMPORAL) {
+  if constexpr (NT) {
     r = __builtin_nontemporal_load(reinterpret_cast<gptr<const R>>(p));
   } else {
     r = *reinterpret_cast<gptr<const R>>(p);
@@ -91,12 +88,8 @@ __device__ __forceinline__ Arr<T, N> ldv(gptr<const T> p) {
 template <typename T, int N>
 __device__ __forceinline__ void stv(gptr<T> p, const Arr<T, N>& a) {
   typedef typename Raw<(int)sizeof(T) * N, (int)alignof(T)>::type R;
-#if HVDHIP_NONTEMPORAL
   __builtin_nontemporal_store(__builtin_bit_cast(typename RawSel<(int)sizeof(T) * N>::type, a),
                               reinterpret_cast<gptr<R>>(p));
-#else
-  *reinterpret_cast<gptr<R>>(p) = __builtin_bit_cast(typename RawSel<(int)sizeof(T) * N>::type, a);
-#endif
 }
 
 // Loads of one-byte elements.  The compiler drops the non-temporal hint from a vector load that
@@ -166,10 +159,9 @@ __device__ __forceinline__ void stw(const Window& w, uint32_t off, const Arr<T, 
     stw<ST, T, N / 2>(w, off + 16, hi);
   } else if constexpr (ST == kStoreWT) {
     typedef typename RawSel<(int)sizeof(T) * N>::type R;
-#ifndef HVDHIP_WT_AUX
-#define HVDHIP_WT_AUX (1 | 16)  // sc0 | sc1
-#endif
-    constexpr int kScopeBits = HVDHIP_WT_AUX;
+    // sc0 | sc1.  (sc1 alone measures the same, no bit at all -- plain write-back -- gains a third
+    // as much, and sc1 with nt loses 5 % against non-temporal stores.)
+    constexpr int kScopeBits = 1 | 16;
     const R r = __builtin_bit_cast(R, a);
     if constexpr (sizeof(T) * N == 16) {
       __builtin_amdgcn_raw_buffer_store_b128(r, w.rsrc, (int)off, 0, kScopeBits);

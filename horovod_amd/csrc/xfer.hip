@@ -35,8 +35,6 @@
 #include <mutex>
 #include <unordered_map>
 
-#include <hip/hip_ext.h>
-
 #include "internal.h"
 #include "vecmem.h"
 
@@ -134,10 +132,7 @@ struct UnpackF16F32 {
   }
 };
 
-#ifndef HVDHIP_XFER_UNROLL
-#define HVDHIP_XFER_UNROLL 4
-#endif
-constexpr int kUnroll = HVDHIP_XFER_UNROLL;  // 16-byte loads in flight per lane
+constexpr int kUnroll = 4;  // 16-byte loads in flight per lane, for chunks of more than one vector per lane
 
 // Streams n elements from src to dst through Op::f with the whole workgroup.
 template <class Op, int ST>
@@ -237,14 +232,10 @@ int launch_xfer(const DevTables& t, uint64_t base, typename Op::P p, hipStream_t
   const Stores family = MODE == kDirect ? (gathers ? Stores::kPack : Stores::kDirect)
                         : MODE == kPack ? (converting ? Stores::kPackNarrowing : Stores::kPack)
                                         : (converting ? Stores::kUnpackWidening : Stores::kUnpack);
-  with_store_policy(family, [&](auto st) {
-    if (completion)
-      hipExtLaunchKernelGGL((xfer_k<Op, MODE, decltype(st)::value>), dim3(t.nchunks), dim3(kWG), 0, stream, nullptr,
-                            completion, 0, t.chunks, base, p);
-    else
-      launch(xfer_k<Op, MODE, decltype(st)::value>, t.nchunks, stream, t.chunks, base, p);
+  const hipError_t status = with_store_policy(family, [&](auto st) {
+    return launch_with(completion, xfer_k<Op, MODE, decltype(st)::value>, t.nchunks, stream, t.chunks, base, p);
   });
-  HVDHIP_CHECK_LAUNCH("xfer_k");
+  HVDHIP_CHECK_LAUNCH("xfer_k", status);
   return 0;
 }
 
@@ -295,10 +286,11 @@ int launch_contig(const void* in, void* out, int64_t n, typename Op::P p, hipStr
     const uint64_t slice = std::min<uint64_t>(left, kMaxWorkgroups * tile);
     const uint32_t blocks = (uint32_t)((slice + tile - 1) / tile);
     const XcdOrder order = xcd_order(blocks, chunk_bytes(Family::kXfer));
-    with_store_policy(Stores::kContig, [&](auto st) {
-      launch(contig_k<Op, decltype(st)::value>, blocks, stream, src, dst, slice, tile, order.shift, order.ordered, p);
+    const hipError_t status = with_store_policy(Stores::kContig, [&](auto st) {
+      return launch(contig_k<Op, decltype(st)::value>, blocks, stream, src, dst, slice, tile, order.shift,
+                    order.ordered, p);
     });
-    HVDHIP_CHECK_LAUNCH("contig_k");
+    HVDHIP_CHECK_LAUNCH("contig_k", status);
     src += slice;
     dst += slice;
     left -= slice;
@@ -464,9 +456,12 @@ int acquire_buf(CopyCache& c, size_t bytes, TableBuf* out) {
 
 // Takes the least recently used entry out of the cache.  Nothing is waited for: an event goes
 // behind whatever each stream that used the table holds now, and the buffers are retired with
-// those events.  A stream that no longer exists cannot take an event; its work is then waited
-// for with the rest of the device (a stream destroyed through hvdhip_stream_destroy has been
-// taken off every entry first, so this is left to foreign streams that were destroyed).
+// those events.  Streams that were given up through hvdhip_stream_destroy or hvdhip_stream_forget
+// have been taken off every entry first.  What is left is a caller's own stream that was destroyed
+// without either call; the contract asks for it to have been idle then.  If the runtime rejects the
+// handle, the rest of the device is waited for; if another stream has since been created at the
+// same address, the event lands behind that stream's work, which is later than needed and
+// harmless, because the old stream's reads had completed before it went away.
 int evict_one(CopyCache& c) {
   auto victim = std::prev(c.lru.end());
   Retired r;

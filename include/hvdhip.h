@@ -121,6 +121,15 @@ int hvdhip_set_device(int device);
  * priority (the reference asks for the greatest priority). */
 int hvdhip_stream_create(void** stream);
 int hvdhip_stream_destroy(void* stream);
+/* For a stream that the caller created itself (the framework's, or hipStreamCreate) and is about
+ * to destroy: waits for the stream, then drops what the library remembers about it -- the copy
+ * tables that launches on it have read (hvdhip_batched_*), its pooled events and the single-layer
+ * Adasum plans made for it (hvdhip_adasum_dot_and_norm_sqrds).  hvdhip_stream_destroy does the
+ * same for the library's own streams.  A caller's stream that is destroyed without this call
+ * must have been idle, and the library then falls back to waiting for the whole device when it
+ * next retires a table that the stream had read.  No counterpart in the reference, which keeps
+ * its streams for the life of the process (ops/gpu_operations.cc:30-39). */
+int hvdhip_stream_forget(void* stream);
 /* GPUContext::StreamSynchronize, ops/cuda_operations.cc:178-180. */
 int hvdhip_stream_synchronize(void* stream);
 /* The framework's ready event is waited for on the Horovod stream, without a

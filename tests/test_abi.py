@@ -128,3 +128,16 @@ def test_more_argument_errors_are_caught_before_the_device_is_touched():
     assert L.hvdhip_memcpy_async(None, None, 0, 9, None) == -1
     for code in (-1, -2, -3, -4, 1, 2, 700):
         assert L.hvdhip_error_string(code)
+
+
+def test_shipped_library_reads_no_tuning_settings():
+    """The chunk size and the store-policy table are fixed in the shipped library; only the tuning
+    build (-DHVDHIP_TUNING, loaded by tests through HVDHIP_LIBRARY) looks at the environment for
+    them.  HVDHIP_EVENT_SYSTEM_FENCE is a documented user setting and stays."""
+    lib_dir = os.path.join(ROOT, "horovod_amd", "lib")
+    shipped = open(os.path.join(lib_dir, "libhvdhip.so"), "rb").read()
+    tuning = open(os.path.join(lib_dir, "libhvdhip_tuning.so"), "rb").read()
+    for name in (b"HVDHIP_CHUNK_BYTES", b"HVDHIP_WRITE_THROUGH"):
+        assert name not in shipped
+        assert name in tuning
+    assert b"HVDHIP_EVENT_SYSTEM_FENCE" in shipped

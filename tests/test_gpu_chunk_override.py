@@ -1,5 +1,7 @@
 """Library settings that are read from the environment once per process, exercised in child
-processes.
+processes.  The chunk size and the store-policy mask are tuning settings that only
+libhvdhip_tuning.so reads (the same sources built with -DHVDHIP_TUNING; the shipped library reads
+neither): the child processes load that build through HVDHIP_LIBRARY.
 
 The kernels' multi-vector (unrolled) inner loops only run when a workgroup's chunk holds more
 than 1,024 vectors; the default 4 KiB chunks never reach them for transfers: the pack / scale /
@@ -20,10 +22,11 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+TUNING = os.path.join(ROOT, "horovod_amd", "lib", "libhvdhip_tuning.so")
 
 
 def test_parity_with_64_kib_chunks(gpu):
-    env = dict(os.environ, HVDHIP_CHUNK_BYTES="65536")
+    env = dict(os.environ, HVDHIP_CHUNK_BYTES="65536", HVDHIP_LIBRARY=TUNING)
     cmd = [sys.executable, "-m", "pytest", "-q", "-x", "-m", "gpu", "--timeout", "300", "--timeout-method", "thread",
            os.path.join(ROOT, "tests", "test_gpu_pack.py"), os.path.join(ROOT, "tests", "test_gpu_scale_reduce.py"),
            os.path.join(ROOT, "tests", "test_gpu_adasum.py"), "-p", "no:cacheprovider"]
@@ -35,7 +38,7 @@ def test_parity_with_64_kib_chunks(gpu):
 
 @pytest.mark.parametrize("mask", ["0", "0x1ff"])
 def test_parity_with_every_kernel_family_on_one_store_policy(gpu, mask):
-    env = dict(os.environ, HVDHIP_WRITE_THROUGH=mask)
+    env = dict(os.environ, HVDHIP_WRITE_THROUGH=mask, HVDHIP_LIBRARY=TUNING)
     files = ["test_gpu_pack.py", "test_gpu_scale_reduce.py", "test_gpu_adasum.py", "test_gpu_configs.py"]
     cmd = [sys.executable, "-m", "pytest", "-q", "-x", "-m", "gpu", "--timeout", "300", "--timeout-method", "thread"] + \
           [os.path.join(ROOT, "tests", f) for f in files] + ["-p", "no:cacheprovider"]
