@@ -1,6 +1,15 @@
 // adapter_capi.cc -- a small C surface over the adapter classes so that the
-// Python tests can drive them (exceptions are turned into a message buffer).
+// Python tests and the benchmark can drive them (exceptions are turned into a message buffer).
+//
+// The harness plays the part of Horovod's background thread: the caller's thread queues one
+// response after the other with GPUAllreduce::Execute, which returns as soon as the kernels
+// are launched; the adapter's finalizer threads wait for each response's events and call
+// the entries' callbacks, which the harness counts per response.
+#include <chrono>
+#include <condition_variable>
 #include <cstring>
+#include <deque>
+#include <mutex>
 #include <stdexcept>
 
 #include "hvd_hip_adapter.h"
@@ -8,11 +17,36 @@
 using namespace horovod::common;
 
 namespace {
+double now_s() {
+  return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+// One queued response as the harness sees it.
+struct Op {
+  int pending = 0;           // entries whose callback has not run yet
+  bool failed = false;
+  std::string reason;
+  double queued_at = 0;      // Execute was called
+  double returned_at = 0;    // Execute returned (kernels launched, completion handed over)
+  double completed_at = 0;   // the last entry's callback ran
+};
+
+// A response whose entries are kept between calls, so that a benchmark loop pays for the
+// launch and not for rebuilding the entry list.
+struct Prepared {
+  std::vector<TensorTableEntry> entries;
+};
+
 struct Harness {
   GPUContext context;
   GlobalState state;
   GPUAllreduce* allreduce = nullptr;
   AdasumGPU* adasum = nullptr;
+  std::mutex mu;
+  std::condition_variable done;
+  std::deque<Op> ops;  // index = ticket; a deque so that queued entries stay where they are
+  int completed = 0;
+  std::vector<Prepared> prepared;
 };
 
 int report(const std::exception& e, char* err, size_t errlen) {
@@ -22,26 +56,114 @@ int report(const std::exception& e, char* err, size_t errlen) {
   }
   return -1;
 }
+
+int report(const std::string& reason, char* err, size_t errlen) {
+  if (err && errlen) {
+    std::strncpy(err, reason.c_str(), errlen - 1);
+    err[errlen - 1] = 0;
+  }
+  return -1;
+}
+
+// Queues one response and returns its ticket.
+int queue_response(Harness* h, std::vector<TensorTableEntry>& entries, double prescale, double postscale,
+                   const void* const* peers, int npeers) {
+  int ticket;
+  {
+    std::lock_guard<std::mutex> guard(h->mu);
+    ticket = (int)h->ops.size();
+    h->ops.emplace_back();
+    h->ops.back().pending = (int)entries.size();
+    h->ops.back().queued_at = now_s();
+  }
+  for (auto& e : entries) {
+    e.callback = [h, ticket](const Status& status) {
+      // what a framework's callback does with asynchronous completion: its own stream (here the
+      // null stream) waits for the event (horovod/torch/mpi_ops_v2.cc:110-116)
+      if (status.event.event) hvdhip_stream_wait_event(nullptr, *status.event.event);
+      std::lock_guard<std::mutex> guard(h->mu);
+      Op& op = h->ops[(size_t)ticket];
+      if (!status.ok() && !op.failed) {
+        op.failed = true;
+        op.reason = status.reason();
+      }
+      if (--op.pending == 0) {
+        op.completed_at = now_s();
+        ++h->completed;
+        h->done.notify_all();
+      }
+    };
+  }
+  std::vector<const void*> p(peers, peers + npeers);
+  try {
+    h->allreduce->Execute(entries, prescale, postscale, p);
+  } catch (...) {
+    // nothing was handed to a finalizer thread: the response is over, with no callbacks to come
+    std::lock_guard<std::mutex> guard(h->mu);
+    Op& op = h->ops[(size_t)ticket];
+    op.pending = 0;
+    op.failed = true;
+    op.completed_at = now_s();
+    ++h->completed;
+    throw;
+  }
+  std::lock_guard<std::mutex> guard(h->mu);
+  h->ops[(size_t)ticket].returned_at = now_s();
+  return ticket;
+}
+
+int wait_ticket(Harness* h, int ticket, char* err, size_t errlen) {
+  std::unique_lock<std::mutex> lock(h->mu);
+  if (ticket < 0 || (size_t)ticket >= h->ops.size()) return report(std::string("unknown ticket"), err, errlen);
+  h->done.wait(lock, [&] { return h->ops[(size_t)ticket].pending == 0; });
+  const Op& op = h->ops[(size_t)ticket];
+  return op.failed ? report(op.reason, err, errlen) : 0;
+}
+
+void fill_entries(std::vector<TensorTableEntry>& entries, const void* const* tensors, void* const* outputs,
+                  const int64_t* counts, int n, int dtype, int buffer_dtype) {
+  entries.resize((size_t)n);
+  for (int i = 0; i < n; ++i) {
+    entries[(size_t)i].tensor_name = "t" + std::to_string(i);
+    entries[(size_t)i].tensor_data = tensors[i];
+    entries[(size_t)i].output_data = outputs[i];
+    entries[(size_t)i].num_elements = counts[i];
+    entries[(size_t)i].dtype = (DataType)dtype;
+    entries[(size_t)i].buffer_dtype = buffer_dtype;
+    entries[(size_t)i].device = 0;
+  }
+}
 }  // namespace
 
 extern "C" {
 
-void* hvd_adapter_create(int num_streams, int batch_d2d_memcopies, int enable_async_completion, int elastic,
-                         void* const* fusion_buffers) {
+// finalizer_threads: threads that wait for queued responses (the reference creates one per stream
+// slot, common/operations.cc:449); 0 runs every completion on the calling thread.
+void* hvd_adapter_create_ex(int num_streams, int batch_d2d_memcopies, int enable_async_completion, int elastic,
+                            void* const* fusion_buffers, int finalizer_threads) {
   Harness* h = new Harness();
   h->state.num_nccl_streams = num_streams;
   h->state.batch_d2d_memcopies = batch_d2d_memcopies != 0;
   h->state.enable_async_completion = enable_async_completion != 0;
   h->state.elastic_enabled = elastic != 0;
   for (int i = 0; i < num_streams; ++i) h->state.fusion_buffer.push_back(fusion_buffers[i]);
+  h->context.streams.resize((size_t)num_streams);
+  if (finalizer_threads > 0) h->context.finalizer_thread_pool.create(finalizer_threads);
   h->allreduce = new GPUAllreduce(&h->context, &h->state);
   h->adasum = new AdasumGPU(&h->context);
   return h;
 }
 
+void* hvd_adapter_create(int num_streams, int batch_d2d_memcopies, int enable_async_completion, int elastic,
+                         void* const* fusion_buffers) {
+  return hvd_adapter_create_ex(num_streams, batch_d2d_memcopies, enable_async_completion, elastic, fusion_buffers,
+                               num_streams);
+}
+
 void hvd_adapter_destroy(void* handle) {
   Harness* h = static_cast<Harness*>(handle);
   if (!h) return;
+  h->context.finalizer_thread_pool.reset();  // the callbacks of queued responses run before the harness goes
   delete h->allreduce;
   delete h->adasum;
   delete h;  // the context's destructor gives its streams back
@@ -58,28 +180,96 @@ int hvd_adapter_allreduce(void* handle, const void* const* tensors, void* const*
                                     npeers, err, errlen);
 }
 
-// buffer_dtype: the dtype of the fusion buffer and of the peers' buffers (-1: that of the tensors).
-int hvd_adapter_allreduce_wire(void* handle, const void* const* tensors, void* const* outputs,
-                               const int64_t* counts, int n, int dtype, int buffer_dtype, double prescale,
-                               double postscale, const void* const* peers, int npeers, char* err, size_t errlen) {
+// Queues one response and returns its ticket (>= 0) as soon as GPUAllreduce::Execute has
+// returned, or -1 with the exception's text.  buffer_dtype: the dtype of the fusion buffer and of
+// the peers' buffers (-1: that of the tensors).
+int hvd_adapter_allreduce_async(void* handle, const void* const* tensors, void* const* outputs,
+                                const int64_t* counts, int n, int dtype, int buffer_dtype, double prescale,
+                                double postscale, const void* const* peers, int npeers, char* err, size_t errlen) {
   Harness* h = static_cast<Harness*>(handle);
   try {
-    std::vector<TensorTableEntry> entries((size_t)n);
-    for (int i = 0; i < n; ++i) {
-      entries[(size_t)i].tensor_name = "t" + std::to_string(i);
-      entries[(size_t)i].tensor_data = tensors[i];
-      entries[(size_t)i].output_data = outputs[i];
-      entries[(size_t)i].num_elements = counts[i];
-      entries[(size_t)i].dtype = (DataType)dtype;
-      entries[(size_t)i].buffer_dtype = buffer_dtype;
-      entries[(size_t)i].device = 0;
-    }
-    std::vector<const void*> p(peers, peers + npeers);
-    h->allreduce->Execute(entries, prescale, postscale, p);
-    return 0;
+    std::vector<TensorTableEntry> entries;
+    fill_entries(entries, tensors, outputs, counts, n, dtype, buffer_dtype);
+    return queue_response(h, entries, prescale, postscale, peers, npeers);
   } catch (const std::exception& e) {
     return report(e, err, errlen);
   }
+}
+
+// The same, waiting for the response's callbacks before it returns: 0, or -1 with the text of
+// the exception or of the failed Status.
+int hvd_adapter_allreduce_wire(void* handle, const void* const* tensors, void* const* outputs,
+                               const int64_t* counts, int n, int dtype, int buffer_dtype, double prescale,
+                               double postscale, const void* const* peers, int npeers, char* err, size_t errlen) {
+  int ticket = hvd_adapter_allreduce_async(handle, tensors, outputs, counts, n, dtype, buffer_dtype, prescale,
+                                           postscale, peers, npeers, err, errlen);
+  if (ticket < 0) return -1;
+  return wait_ticket(static_cast<Harness*>(handle), ticket, err, errlen);
+}
+
+// Keeps a response's entry list in the harness; returns its id.
+int hvd_adapter_prepare(void* handle, const void* const* tensors, void* const* outputs, const int64_t* counts,
+                        int n, int dtype, int buffer_dtype) {
+  Harness* h = static_cast<Harness*>(handle);
+  h->prepared.emplace_back();
+  fill_entries(h->prepared.back().entries, tensors, outputs, counts, n, dtype, buffer_dtype);
+  return (int)h->prepared.size() - 1;
+}
+
+// Queues a prepared response; returns its ticket or -1.
+int hvd_adapter_execute_prepared(void* handle, int id, double prescale, double postscale,
+                                 const void* const* peers, int npeers, char* err, size_t errlen) {
+  Harness* h = static_cast<Harness*>(handle);
+  try {
+    if (id < 0 || (size_t)id >= h->prepared.size()) throw std::logic_error("unknown prepared response");
+    return queue_response(h, h->prepared[(size_t)id].entries, prescale, postscale, peers, npeers);
+  } catch (const std::exception& e) {
+    return report(e, err, errlen);
+  }
+}
+
+int hvd_adapter_wait(void* handle, int ticket, char* err, size_t errlen) {
+  return wait_ticket(static_cast<Harness*>(handle), ticket, err, errlen);
+}
+
+// Waits for every response queued so far; -1 with the first failure's text if one failed.
+int hvd_adapter_wait_all(void* handle, char* err, size_t errlen) {
+  Harness* h = static_cast<Harness*>(handle);
+  std::unique_lock<std::mutex> lock(h->mu);
+  h->done.wait(lock, [&] { return h->completed == (int)h->ops.size(); });
+  for (const Op& op : h->ops)
+    if (op.failed) return report(op.reason, err, errlen);
+  return 0;
+}
+
+// Responses whose callbacks have all run.
+int hvd_adapter_completed(void* handle) {
+  Harness* h = static_cast<Harness*>(handle);
+  std::lock_guard<std::mutex> guard(h->mu);
+  return h->completed;
+}
+
+// Steady-clock seconds at which Execute was called for the ticket, returned, and the last callback
+// ran (0 while that has not happened).
+int hvd_adapter_op_times(void* handle, int ticket, double* queued_at, double* returned_at, double* completed_at) {
+  Harness* h = static_cast<Harness*>(handle);
+  std::lock_guard<std::mutex> guard(h->mu);
+  if (ticket < 0 || (size_t)ticket >= h->ops.size()) return -1;
+  const Op& op = h->ops[(size_t)ticket];
+  *queued_at = op.queued_at;
+  *returned_at = op.returned_at;
+  *completed_at = op.completed_at;
+  return 0;
+}
+
+// Forgets the finished responses' bookkeeping (tickets start again at 0); all must have completed.
+int hvd_adapter_reset_tickets(void* handle) {
+  Harness* h = static_cast<Harness*>(handle);
+  std::lock_guard<std::mutex> guard(h->mu);
+  if (h->completed != (int)h->ops.size()) return -1;
+  h->ops.clear();
+  h->completed = 0;
+  return 0;
 }
 
 // Switches the timeline hooks on or off.
@@ -91,6 +281,7 @@ void hvd_adapter_set_timeline(void* handle, int on) {
 int hvd_adapter_timeline(void* handle, char* out, size_t outlen) {
   Harness* h = static_cast<Harness*>(handle);
   std::string s;
+  std::lock_guard<std::mutex> guard(h->state.timeline_mutex);
   for (auto& a : h->state.timeline_activities) s += (s.empty() ? "" : ",") + a;
   h->state.timeline_activities.clear();
   std::strncpy(out, s.c_str(), outlen - 1);

@@ -1,6 +1,7 @@
 // hvd_hip_adapter.cc -- see hvd_hip_adapter.h.  Host code; links only libhvdhip.so.
 #include "hvd_hip_adapter.h"
 
+#include <algorithm>
 #include <stdexcept>
 #include <thread>
 
@@ -20,12 +21,68 @@ const std::string& DataType_Name(DataType value) {
   return ((int)value >= 0 && (int)value <= 9) ? names[(int)value] : unknown;
 }
 
+// ---------------------------------------------------------------- ThreadPool
+
+ThreadPool::~ThreadPool() { reset(); }
+
+void ThreadPool::create(int num_threads) {
+  reset();
+  {
+    std::lock_guard<std::mutex> guard(mutex_);
+    stopping_ = false;
+  }
+  for (int i = 0; i < num_threads; ++i) threads_.emplace_back([this] { loop(); });
+}
+
+void ThreadPool::execute(std::function<void(void)> f) {
+  {
+    std::lock_guard<std::mutex> guard(mutex_);
+    queue_.push_back(std::move(f));
+  }
+  work_.notify_one();
+}
+
+void ThreadPool::loop() {
+  std::unique_lock<std::mutex> lock(mutex_);
+  for (;;) {
+    work_.wait(lock, [this] { return stopping_ || !queue_.empty(); });
+    if (queue_.empty()) return;  // stopping, and nothing left to run
+    std::function<void(void)> task = std::move(queue_.front());
+    queue_.pop_front();
+    ++busy_;
+    lock.unlock();
+    task();
+    task = nullptr;  // what the task captured goes before the pool reads as idle
+    lock.lock();
+    --busy_;
+    idle_.notify_all();
+  }
+}
+
+void ThreadPool::wait_idle() {
+  std::unique_lock<std::mutex> lock(mutex_);
+  if (threads_.empty()) return;
+  idle_.wait(lock, [this] { return queue_.empty() && busy_ == 0; });
+}
+
+void ThreadPool::reset() {
+  {
+    std::lock_guard<std::mutex> guard(mutex_);
+    stopping_ = true;
+  }
+  work_.notify_all();
+  for (auto& t : threads_) t.join();
+  threads_.clear();
+}
+
 // ---------------------------------------------------------------- GPUContext
 
 GPUContext::GPUContext() {}
 // The reference keeps its streams for the life of the process; a context that can be created
-// and dropped many times (tests, benchmarks) gives them back.
+// and dropped many times (tests, benchmarks) gives them back, after the finalizer threads have
+// run what was handed to them.
 GPUContext::~GPUContext() {
+  finalizer_thread_pool.reset();
   for (auto& per_device : streams)
     for (auto& kv : per_device)
       if (kv.second) hvdhip_stream_destroy(kv.second);
@@ -77,18 +134,24 @@ void GPUContext::WaitForEvents(std::queue<std::pair<std::string, Event>>& event_
       while (true) {
         int done = 0;
         int rc = hvdhip_event_query(*event.event, &done);
-        if (rc != 0) throw std::logic_error(std::string("hipEventQuery failed: ") + hvdhip_error_string(rc));
+        if (rc != 0) {
+          hvdhip_event_release(event.stream, *event.event);  // a failed wait still gives its event back
+          throw std::logic_error(std::string("hipEventQuery failed: ") + hvdhip_error_string(rc));
+        }
         if (done) break;
         if (error_check_callback) error_check_callback();
         std::this_thread::yield();
       }
     } else {
       int rc = hvdhip_event_synchronize(*event.event);
-      if (rc != 0) throw std::logic_error(std::string("hipEventSynchronize failed: ") + hvdhip_error_string(rc));
+      if (rc != 0) {
+        hvdhip_event_release(event.stream, *event.event);
+        throw std::logic_error(std::string("hipEventSynchronize failed: ") + hvdhip_error_string(rc));
+      }
       if (error_check_callback) error_check_callback();
     }
     // timeline.ActivityStartAll(entries, name) ... ActivityEndAll(entries) bracket the wait
-    if (name != "" && timeline_activities) timeline_activities->push_back(name);
+    if (name != "" && timeline_activities) timeline_activities->push_back(name);  // the caller's own vector
     ErrorCheck("ReleaseGpuEvent", hvdhip_event_release(event.stream, *event.event));
   }
 }
@@ -160,21 +223,65 @@ void* GPUOpContext::QueueCompletionEvent() {
   return *event.event;
 }
 
-void GPUOpContext::FinalizeGPUQueue(std::vector<TensorTableEntry>& entries,
-                                    const std::function<void()>& error_check_callback) {
+Status GPUOpContext::FinalizeGPUQueue(std::vector<TensorTableEntry>& entries,
+                                      const std::function<void()>& error_check_callback) {
+  // A completion marker on the stream instead of a blocking stream synchronisation on this thread.
   if (!global_state_->enable_async_completion && !completion_queued_)
     gpu_context_->RecordEvent(event_queue, "", *stream);
-  gpu_context_->SetDevice(entries[0].device);
-  if (!global_state_->enable_async_completion || global_state_->timeline_initialized) {
-    // with the timeline on, events are waited for on the host for accurate timings (ops/gpu_operations.cc:77-80)
-    gpu_context_->WaitForEvents(event_queue, error_check_callback, global_state_->elastic_enabled,
-                                &global_state_->timeline_activities);
-  } else {
-    gpu_context_->ClearEvents(event_queue);
-    Event event = gpu_context_->RecordEvent(*stream);  // handed to the framework in Status.event
-    gpu_context_->ReleaseEvent(event);
-  }
+
+  // Everything the completion needs travels by value: this context is reused by the next response
+  // while a finalizer thread still works on this one.
+  GPUContext* gpu_context = gpu_context_;
+  GlobalState* global_state = global_state_;
+  const int device = entries[0].device;
+  const bool elastic = global_state_->elastic_enabled;
+  const bool async_completion = global_state_->enable_async_completion;
+  const bool timeline = global_state_->timeline_initialized;
+  gpuStream_t current_stream = *stream;
+  auto events = event_queue;
+  auto finalize = [gpu_context, global_state, device, elastic, async_completion, timeline, current_stream, events,
+                   entries, error_check_callback]() mutable {
+    Status status = Status::OK();
+    try {
+      gpu_context->SetDevice(device);  // ops/gpu_operations.cc:75: the thread has no device of its own yet
+      if (!async_completion || timeline) {
+        // with the timeline on, events are waited for on the host for accurate timings (ops/gpu_operations.cc:77-80)
+        std::vector<std::string> activities;
+        gpu_context->WaitForEvents(events, error_check_callback, elastic, &activities);
+        if (!activities.empty()) {
+          std::lock_guard<std::mutex> guard(global_state->timeline_mutex);
+          for (auto& a : activities) global_state->timeline_activities.push_back(a);
+        }
+      } else {
+        gpu_context->ClearEvents(events);
+        status.event = gpu_context->RecordEvent(current_stream);  // the framework's stream waits for this one
+      }
+    } catch (const std::exception& e) {
+      // an exception must not leave a finalizer thread; the entries learn of it as the reference's
+      // background loop reports a failed op (common/operations.cc:291-305)
+      Event recorded = status.event;
+      status = Status::UnknownError(e.what());
+      status.event = recorded;
+      try {
+        gpu_context->ClearEvents(events);  // the events behind the one that failed go back to the pool
+      } catch (const std::exception&) {
+      }
+    }
+    for (auto& e : entries) e.FinishWithCallback(status);
+    if (status.event.event) {
+      try {
+        gpu_context->ReleaseEvent(status.event);
+      } catch (const std::exception&) {
+      }
+    }
+  };
+  if (gpu_context_->finalizer_thread_pool.size() > 0)
+    gpu_context_->finalizer_thread_pool.execute(std::move(finalize));
+  else
+    finalize();
+
   global_state_->current_nccl_stream = (global_state_->current_nccl_stream + 1) % global_state_->num_nccl_streams;
+  return Status::InProgress();
 }
 
 // -------------------------------------------------------------- GPUAllreduce
@@ -311,8 +418,8 @@ void GPUAllreduce::ScaleBuffer(double scale_factor, const std::vector<TensorTabl
                                 Stream(entries));
 }
 
-void GPUAllreduce::Execute(std::vector<TensorTableEntry>& entries, double prescale_factor,
-                           double postscale_factor, const std::vector<const void*>& peers) {
+Status GPUAllreduce::Execute(std::vector<TensorTableEntry>& entries, double prescale_factor,
+                             double postscale_factor, const std::vector<const void*>& peers) {
   auto& first_entry = entries[0];
   gpu_op_context_.InitGPU(entries);
   gpu_op_context_.InitGPUQueue(entries);
@@ -357,7 +464,7 @@ void GPUAllreduce::Execute(std::vector<TensorTableEntry>& entries, double presca
   } else if (postscale_factor != 1.0) {
     ScaleBuffer(postscale_factor, entries, buffer_data, buffer_data, first_entry.num_elements);
   }
-  gpu_op_context_.FinalizeGPUQueue(entries);
+  return gpu_op_context_.FinalizeGPUQueue(entries);
 }
 
 // --------------------------------------------------------------- GPUAllgather

@@ -6,6 +6,9 @@
 // reference's):
 //   GPUContext          ops/gpu_operations.h:44-106, impl ops/cuda_operations.cc:28-210
 //   GPUOpContext        ops/gpu_operations.h:108-137, ops/gpu_operations.cc:27-106
+//   ThreadPool          common/thread_pool.h:27-43 (the finalizer threads, one per stream slot,
+//                       common/operations.cc:449)
+//   Status              common/common.h:192-212
 //   GPUAllreduce hooks  ops/gpu_operations.h:139-172, ops/gpu_operations.cc:118-339
 //   Adasum dispatch     ops/adasum/adasum.h:101-140,344-410
 //   FuseResponses       common/controller.cc:793-866
@@ -19,14 +22,18 @@
 #ifndef HVD_HIP_ADAPTER_H
 #define HVD_HIP_ADAPTER_H
 
+#include <condition_variable>
 #include <cstddef>
 #include <cstdint>
+#include <deque>
 #include <functional>
 #include <list>
 #include <map>
 #include <memory>
+#include <mutex>
 #include <queue>
 #include <string>
+#include <thread>
 #include <unordered_map>
 #include <utility>
 #include <vector>
@@ -52,8 +59,37 @@ typedef void* gpuStream_t;
 #define MEMCPY_OUT_FUSION_BUFFER "MEMCPY_OUT_FUSION_BUFFER"
 #define NCCL_ALLREDUCE "NCCL_ALLREDUCE"
 
+// common/common.h:181-189
+struct Event {
+  std::shared_ptr<void*> event;
+  gpuStream_t stream = nullptr;
+};
+
+// common/common.h:157,192-212
+enum StatusType { OK, UNKNOWN_ERROR, PRECONDITION_ERROR, ABORTED, INVALID_ARGUMENT, IN_PROGRESS };
+class Status {
+public:
+  Status() {}
+  static Status OK() { return Status(); }
+  static Status UnknownError(const std::string& message) { return Status(UNKNOWN_ERROR, message); }
+  static Status InProgress() { return Status(IN_PROGRESS, ""); }
+  bool ok() const { return type_ == StatusType::OK; }
+  bool in_progress() const { return type_ == IN_PROGRESS; }
+  StatusType type() const { return type_; }
+  const std::string& reason() const { return reason_; }
+  // With asynchronous completion: recorded behind the response on its stream; the framework's
+  // callback makes its own stream wait for it (horovod/torch/mpi_ops_v2.cc:110-116).
+  Event event;
+
+private:
+  Status(StatusType type, std::string reason) : type_(type), reason_(std::move(reason)) {}
+  StatusType type_ = StatusType::OK;
+  std::string reason_;
+};
+typedef std::function<void(const Status&)> StatusCallback;
+
 // The part of TensorTableEntry (common/common.h:341-374) that the hooks read:
-// tensor->data()/size()/dtype(), output->data(), device.
+// tensor->data()/size()/dtype(), output->data(), device, callback.
 struct TensorTableEntry {
   std::string tensor_name;
   const void* tensor_data = nullptr;
@@ -67,12 +103,40 @@ struct TensorTableEntry {
   // left at its default the entry travels as it is.
   int buffer_dtype = -1;
   DataType wire_dtype() const { return buffer_dtype < 0 ? dtype : (DataType)buffer_dtype; }
+  // Called from a finalizer thread once the response has completed (or, with asynchronous
+  // completion, once its last work has been queued); may be empty (common/common.cc:202-208).
+  StatusCallback callback;
+  void FinishWithCallback(const Status& status) const {
+    if (callback) callback(status);
+  }
 };
 
-// common/common.h:181-189
-struct Event {
-  std::shared_ptr<void*> event;
-  gpuStream_t stream = nullptr;
+// The finalizer threads: the background thread hands the wait for a response's events to one of
+// them and goes on to launch the next response on the next stream slot.  Same surface as the
+// reference's pool (create / execute / reset), plus wait_idle() so that a harness can tell when
+// everything handed over has run.  reset() runs what is still queued before the threads end, so a
+// response whose wait was queued always gets its callbacks.
+class ThreadPool {
+public:
+  ThreadPool() {}
+  ~ThreadPool();
+  ThreadPool(const ThreadPool&) = delete;
+  ThreadPool& operator=(const ThreadPool&) = delete;
+  void create(int num_threads);
+  void execute(std::function<void(void)> f);
+  void reset();
+  void wait_idle();
+  int size() const { return (int)threads_.size(); }
+
+private:
+  void loop();
+  std::mutex mutex_;
+  std::condition_variable work_;   // a task was queued, or the pool is stopping
+  std::condition_variable idle_;   // a task finished
+  std::deque<std::function<void(void)>> queue_;
+  std::vector<std::thread> threads_;
+  int busy_ = 0;
+  bool stopping_ = false;
 };
 
 class GPUContext {
@@ -82,6 +146,10 @@ public:
 
   // One stream per (stream slot, device), created lazily (ops/gpu_operations.cc:30-39).
   std::vector<std::unordered_map<int, gpuStream_t>> streams;
+  // Completion of queued responses (ops/gpu_operations.h:65); created with one thread per stream
+  // slot by whoever owns the context (common/operations.cc:449).  Left without threads,
+  // FinalizeGPUQueue runs the completion on the calling thread.
+  ThreadPool finalizer_thread_pool;
 
   void ErrorCheck(std::string op_name, int gpu_result);
   void RecordEvent(std::queue<std::pair<std::string, Event>>& event_queue, std::string name, gpuStream_t& stream);
@@ -115,7 +183,8 @@ struct GlobalState {
   // (ops/nccl_operations.cc:173-175,195-197,203-205) and the completed activity names are
   // appended to timeline_activities as the events are waited for.
   bool timeline_initialized = false;
-  std::vector<std::string> timeline_activities;
+  std::vector<std::string> timeline_activities;  // appended to by finalizer threads, under timeline_mutex
+  std::mutex timeline_mutex;
   // One fusion buffer per stream slot (common/fusion_buffer_manager.cc:25); owned by the framework.
   std::vector<void*> fusion_buffer;
 };
@@ -125,10 +194,12 @@ public:
   GPUOpContext(GPUContext* context, GlobalState* global_state);
   void InitGPU(const std::vector<TensorTableEntry>& entries);
   void InitGPUQueue(const std::vector<TensorTableEntry>& entries);
-  // Records the completion event, waits for the queued events (the reference
-  // hands this to a finalizer thread; here it runs inline), rotates the stream slot.
-  void FinalizeGPUQueue(std::vector<TensorTableEntry>& entries,
-                        const std::function<void()>& error_check_callback = nullptr);
+  // Records the completion event, hands the wait for the queued events and the entries'
+  // callbacks to a finalizer thread (ops/gpu_operations.cc:50-99), rotates the stream slot and
+  // returns Status::InProgress() at once, so that the caller can launch the next response on
+  // the next slot while this one runs.
+  Status FinalizeGPUQueue(std::vector<TensorTableEntry>& entries,
+                          const std::function<void()>& error_check_callback = nullptr);
   std::queue<std::pair<std::string, Event>> event_queue;
   gpuStream_t* stream = nullptr;
   // Whether the response's last kernel should carry the completion event itself
@@ -152,9 +223,10 @@ public:
 
   // The op sequence of NCCLAllreduce::Execute (ops/nccl_operations.cc:156-214) with the
   // collective replaced by a local sum with `peers` (device buffers laid out like the
-  // fusion buffer, or like the single tensor).
-  void Execute(std::vector<TensorTableEntry>& entries, double prescale_factor, double postscale_factor,
-               const std::vector<const void*>& peers);
+  // fusion buffer, or like the single tensor).  Returns Status::InProgress() as soon as the
+  // response is queued; every entry's callback is called once it has completed.
+  Status Execute(std::vector<TensorTableEntry>& entries, double prescale_factor, double postscale_factor,
+                 const std::vector<const void*>& peers);
 
   void MemcpyInFusionBuffer(const std::vector<TensorTableEntry>& entries, const void*& fused_input_data,
                             void*& buffer_data, size_t& buffer_len);

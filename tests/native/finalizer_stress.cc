@@ -1,0 +1,302 @@
+// finalizer_stress.cc -- the adapter's host logic (GPUAllreduce::Execute, GPUOpContext::FinalizeGPUQueue,
+// the finalizer ThreadPool, pooled events, callbacks) against the pretend device of fake_hvdhip.cc.
+// Meant to be built with -fsanitize=thread: every scenario must come out right AND race-free.
+// Prints "finalizer ok" when all scenarios pass.
+#include <atomic>
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <mutex>
+#include <set>
+#include <thread>
+#include <vector>
+
+#include "hvd_hip_adapter.h"
+
+using namespace horovod::common;
+
+extern "C" {
+void fake_set_kernel_delay_us(int us);
+void fake_fail_next_event_syncs(int n);
+int fake_events_outstanding();
+int fake_set_device_calls_on_other_threads(void);
+}
+
+#define REQUIRE(cond)                                                     \
+  do {                                                                    \
+    if (!(cond)) {                                                        \
+      std::printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond);         \
+      std::exit(1);                                                       \
+    }                                                                     \
+  } while (0)
+
+namespace {
+
+double now_s() { return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count(); }
+
+// One response's tensors, outputs, peer buffer and what its callbacks saw.
+struct Response {
+  std::vector<std::vector<float>> tensors, outputs;
+  std::vector<float> peer;  // laid out like the fusion buffer (16-byte padded offsets)
+  std::vector<TensorTableEntry> entries;
+  std::atomic<int> callbacks{0};
+  std::atomic<int> failures{0};
+  std::atomic<int> with_event{0};
+  double completed_at = 0;
+  std::thread::id finished_on;
+  std::mutex mu;
+  std::string reason;
+};
+
+void build(Response& r, int seed, const std::vector<int>& counts) {
+  std::srand((unsigned)seed);
+  int64_t off = 0;
+  std::vector<int64_t> offs;
+  for (int c : counts) {
+    offs.push_back(off);
+    off += 16 * ((c * 4 + 15) / 16);
+  }
+  r.peer.assign((size_t)off / 4, 0.f);
+  for (size_t i = 0; i < counts.size(); ++i) {
+    std::vector<float> t((size_t)counts[i]);
+    for (auto& x : t) x = (float)(std::rand() % 2001 - 1000) / 64.f;
+    for (int j = 0; j < counts[i]; ++j) r.peer[(size_t)offs[i] / 4 + (size_t)j] = (float)(std::rand() % 2001 - 1000) / 32.f;
+    r.tensors.push_back(t);
+    r.outputs.emplace_back((size_t)counts[i], -1.f);
+  }
+  r.entries.resize(counts.size());
+  for (size_t i = 0; i < counts.size(); ++i) {
+    TensorTableEntry& e = r.entries[i];
+    e.tensor_name = "r" + std::to_string(seed) + "." + std::to_string(i);
+    e.tensor_data = r.tensors[i].data();
+    e.output_data = r.outputs[i].data();
+    e.num_elements = counts[i];
+    e.dtype = HOROVOD_FLOAT32;
+    Response* rp = &r;
+    e.callback = [rp](const Status& s) {
+      if (!s.ok()) {
+        ++rp->failures;
+        std::lock_guard<std::mutex> g(rp->mu);
+        rp->reason = s.reason();
+      }
+      if (s.event.event) ++rp->with_event;
+      {
+        std::lock_guard<std::mutex> g(rp->mu);
+        rp->completed_at = now_s();
+        rp->finished_on = std::this_thread::get_id();
+      }
+      ++rp->callbacks;
+    };
+  }
+}
+
+void check(const Response& r, const std::vector<int>& counts, float pre, float post, bool with_peer) {
+  int64_t off = 0;
+  for (size_t i = 0; i < counts.size(); ++i) {
+    for (int j = 0; j < counts[i]; ++j) {
+      float v = pre == 1.f ? r.tensors[i][(size_t)j] : pre * r.tensors[i][(size_t)j];
+      if (with_peer) v = v + r.peer[(size_t)off / 4 + (size_t)j];
+      if (post != 1.f) v = post * v;
+      REQUIRE(r.outputs[i][(size_t)j] == v);
+    }
+    off += 16 * ((counts[i] * 4 + 15) / 16);
+  }
+}
+
+struct Rig {
+  GPUContext context;
+  GlobalState state;
+  std::vector<std::vector<char>> buffers;
+  GPUAllreduce* op = nullptr;
+  Rig(int slots, int threads, bool async_completion = false, bool elastic = false, bool timeline = false) {
+    state.num_nccl_streams = slots;
+    state.enable_async_completion = async_completion;
+    state.elastic_enabled = elastic;
+    state.timeline_initialized = timeline;
+    buffers.assign((size_t)slots, std::vector<char>(1 << 20));
+    for (auto& b : buffers) state.fusion_buffer.push_back(b.data());
+    context.streams.resize((size_t)slots);
+    if (threads > 0) context.finalizer_thread_pool.create(threads);
+    op = new GPUAllreduce(&context, &state);
+  }
+  ~Rig() {
+    context.finalizer_thread_pool.reset();
+    delete op;
+  }
+};
+
+void wait_for(const Response& r) {
+  while (r.callbacks.load() < (int)r.entries.size()) std::this_thread::sleep_for(std::chrono::microseconds(50));
+}
+
+// 1. Many responses over two slots: results, one callback per entry, all from finalizer threads.
+void many_responses() {
+  Rig rig(2, 2);
+  const std::vector<int> counts = {5, 1000, 3, 257};
+  const int n = 300;
+  std::vector<Response> rs((size_t)n);
+  for (int i = 0; i < n; ++i) build(rs[(size_t)i], i, counts);
+  for (int i = 0; i < n; ++i) {
+    std::vector<const void*> peers = {rs[(size_t)i].peer.data()};
+    Status s = rig.op->Execute(rs[(size_t)i].entries, 0.125, 0.5, peers);
+    REQUIRE(s.in_progress());
+    REQUIRE(rig.state.current_nccl_stream == (i + 1) % 2);
+  }
+  rig.context.finalizer_thread_pool.wait_idle();
+  std::set<std::thread::id> finishers;
+  for (auto& r : rs) {
+    REQUIRE(r.callbacks == (int)counts.size() && r.failures == 0 && r.with_event == 0);
+    REQUIRE(r.finished_on != std::this_thread::get_id());
+    finishers.insert(r.finished_on);
+    check(r, counts, 0.125f, 0.5f, true);
+  }
+  REQUIRE(finishers.size() <= 2);
+  REQUIRE(fake_set_device_calls_on_other_threads() >= n);  // SetDevice at the top of every finalizer task
+  REQUIRE(fake_events_outstanding() == 0);                 // every pooled event went back
+  REQUIRE(rig.op->cached_plans() == (size_t)128);          // 300 distinct entry lists, bounded cache
+  std::printf("many responses: %d over 2 slots, %zu finalizer thread(s) saw completions\n", n, finishers.size());
+}
+
+// 2. Two consecutive responses on alternating slots are both in flight before either completes, and
+//    run side by side on the pretend device.
+void two_in_flight() {
+  Rig rig(2, 2);
+  const std::vector<int> counts = {64, 64};
+  std::vector<Response> rs(4);
+  for (int i = 0; i < 4; ++i) build(rs[(size_t)i], 1000 + i, counts);
+  // warm-up: plans and streams exist afterwards
+  for (int i = 0; i < 2; ++i) {
+    std::vector<const void*> peers = {rs[(size_t)i].peer.data()};
+    rig.op->Execute(rs[(size_t)i].entries, 1.0, 1.0, peers);
+  }
+  rig.context.finalizer_thread_pool.wait_idle();
+  fake_set_kernel_delay_us(20000);  // 3 kernels of 20 ms per response
+  const double t0 = now_s();
+  double returned[2];
+  for (int i = 2; i < 4; ++i) {
+    std::vector<const void*> peers = {rs[(size_t)i].peer.data()};
+    rig.op->Execute(rs[(size_t)i].entries, 1.0, 1.0, peers);
+    returned[i - 2] = now_s();
+  }
+  REQUIRE(rs[2].callbacks == 0 && rs[3].callbacks == 0);  // neither has completed: both are in flight
+  rig.context.finalizer_thread_pool.wait_idle();
+  fake_set_kernel_delay_us(0);
+  const double total = now_s() - t0;
+  REQUIRE(returned[1] < rs[2].completed_at && returned[1] < rs[3].completed_at);
+  REQUIRE(returned[1] - t0 < 0.030);  // Execute does not wait for the device
+  REQUIRE(total < 0.100);             // 2 x 60 ms of kernels took well under 120 ms: the slots overlapped
+  check(rs[2], counts, 1.f, 1.f, true);
+  check(rs[3], counts, 1.f, 1.f, true);
+  std::printf("two in flight: both Executes returned after %.1f ms, both responses done after %.1f ms\n",
+              (returned[1] - t0) * 1e3, total * 1e3);
+}
+
+// 3. A failure on the finalizer thread reaches every entry's callback as an error Status.
+void failure_reaches_callbacks() {
+  Rig rig(1, 1);
+  const std::vector<int> counts = {10, 20, 30};
+  Response r;
+  build(r, 7, counts);
+  fake_fail_next_event_syncs(1);
+  Status s = rig.op->Execute(r.entries, 1.0, 1.0, {});
+  REQUIRE(s.in_progress());
+  rig.context.finalizer_thread_pool.wait_idle();
+  REQUIRE(r.callbacks == 3 && r.failures == 3);
+  REQUIRE(r.reason.find("hipEventSynchronize failed") != std::string::npos);
+  // the pool goes on working afterwards
+  Response r2;
+  build(r2, 8, counts);
+  rig.op->Execute(r2.entries, 0.5, 1.0, {});
+  rig.context.finalizer_thread_pool.wait_idle();
+  REQUIRE(r2.callbacks == 3 && r2.failures == 0);
+  check(r2, counts, 0.5f, 1.f, false);
+  std::printf("failure: %s\n", r.reason.c_str());
+}
+
+// 4. No finalizer threads: the completion runs on the caller's thread before Execute returns.
+void inline_completion() {
+  Rig rig(2, 0);
+  const std::vector<int> counts = {100, 1};
+  Response r;
+  build(r, 9, counts);
+  std::vector<const void*> peers = {r.peer.data()};
+  Status s = rig.op->Execute(r.entries, 1.0, 0.25, peers);
+  REQUIRE(s.in_progress());
+  REQUIRE(r.callbacks == 2 && r.finished_on == std::this_thread::get_id());
+  check(r, counts, 1.f, 0.25f, true);
+}
+
+// 5. Asynchronous completion: nothing is waited for; the callbacks get an event that has been
+//    recorded behind the response, and the event is released after them.
+void async_completion() {
+  Rig rig(1, 1, /*async_completion=*/true);
+  const std::vector<int> counts = {50, 60};
+  Response r;
+  build(r, 10, counts);
+  fake_set_kernel_delay_us(5000);
+  rig.op->Execute(r.entries, 0.5, 1.0, {});
+  rig.context.finalizer_thread_pool.wait_idle();
+  fake_set_kernel_delay_us(0);
+  REQUIRE(r.callbacks == 2 && r.with_event == 2 && r.failures == 0);
+  REQUIRE(fake_events_outstanding() == 0);
+  rig.context.StreamSynchronize(rig.context.streams[0][0]);
+  check(r, counts, 0.5f, 1.f, false);
+}
+
+// 6. Elastic polling and the timeline's per-stage events, completed on finalizer threads.
+void elastic_and_timeline() {
+  Rig rig(2, 2, false, /*elastic=*/true, /*timeline=*/true);
+  const std::vector<int> counts = {33, 44};
+  std::vector<Response> rs(6);
+  for (int i = 0; i < 6; ++i) {
+    build(rs[(size_t)i], 20 + i, counts);
+    std::vector<const void*> peers = {rs[(size_t)i].peer.data()};
+    rig.op->Execute(rs[(size_t)i].entries, 1.0, 1.0, peers);
+  }
+  rig.context.finalizer_thread_pool.wait_idle();
+  for (auto& r : rs) check(r, counts, 1.f, 1.f, true);
+  std::lock_guard<std::mutex> g(rig.state.timeline_mutex);
+  REQUIRE(rig.state.timeline_activities.size() == 6 * 4);  // QUEUE, MEMCPY_IN, NCCL_ALLREDUCE, MEMCPY_OUT per response
+}
+
+// 7. A pool that is reset with work still queued runs it first; tasks from several producers all run.
+void pool_semantics() {
+  std::atomic<int> ran{0};
+  {
+    ThreadPool pool;
+    pool.create(3);
+    std::vector<std::thread> producers;
+    for (int p = 0; p < 4; ++p)
+      producers.emplace_back([&] {
+        for (int i = 0; i < 500; ++i) pool.execute([&] { ++ran; });
+      });
+    for (auto& t : producers) t.join();
+    pool.execute([&] {
+      std::this_thread::sleep_for(std::chrono::milliseconds(5));
+      ++ran;
+    });
+    pool.reset();
+    REQUIRE(ran == 2001);
+    pool.create(1);  // a pool can be created again after a reset
+    pool.execute([&] { ++ran; });
+    pool.wait_idle();
+    REQUIRE(ran == 2002);
+  }
+  ThreadPool idle;
+  idle.wait_idle();  // no threads: nothing to wait for
+}
+
+}  // namespace
+
+int main() {
+  std::setvbuf(stdout, nullptr, _IONBF, 0);
+  pool_semantics();
+  many_responses();
+  two_in_flight();
+  failure_reaches_callbacks();
+  inline_completion();
+  async_completion();
+  elastic_and_timeline();
+  std::printf("finalizer ok\n");
+  return 0;
+}

@@ -30,6 +30,13 @@ def adapter(gpu):
                                                ctypes.c_double, ctypes.c_void_p, ctypes.c_int, ctypes.c_char_p,
                                                ctypes.c_size_t]
     lib.hvd_adapter_state.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
+    lib.hvd_adapter_create_ex.restype = ctypes.c_void_p
+    lib.hvd_adapter_create_ex.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_int]
+    lib.hvd_adapter_allreduce_async.argtypes = lib.hvd_adapter_allreduce_wire.argtypes
+    lib.hvd_adapter_wait.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t]
+    lib.hvd_adapter_wait_all.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]
+    lib.hvd_adapter_completed.argtypes = [ctypes.c_void_p]
+    lib.hvd_adapter_op_times.argtypes = [ctypes.c_void_p, ctypes.c_int] + [ctypes.POINTER(ctypes.c_double)] * 3
     lib.hvd_adapter_adasum_pairwise.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                                 ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_char_p,
                                                 ctypes.c_size_t]
@@ -47,11 +54,32 @@ def _ptrs(values):
 
 
 class Harness:
-    def __init__(self, lib, gpu, num_streams=2, batch=True, async_completion=False, elastic=False, fb_bytes=1 << 22):
+    def __init__(self, lib, gpu, num_streams=2, batch=True, async_completion=False, elastic=False, fb_bytes=1 << 22,
+                 finalizer_threads=None):
         self.lib = lib
         self.fbs = [gpu.empty(fb_bytes, fill=0xCD) for _ in range(num_streams)]
-        self.h = lib.hvd_adapter_create(num_streams, int(batch), int(async_completion), int(elastic),
-                                        _ptrs([t.data_ptr() for t in self.fbs]))
+        self.h = lib.hvd_adapter_create_ex(num_streams, int(batch), int(async_completion), int(elastic),
+                                           _ptrs([t.data_ptr() for t in self.fbs]),
+                                           num_streams if finalizer_threads is None else finalizer_threads)
+
+    def allreduce_async(self, tensors, outputs, counts, dtype, prescale, postscale, peers=()):
+        """Returns the ticket as soon as GPUAllreduce::Execute has returned."""
+        err = ctypes.create_string_buffer(512)
+        cnt = (ctypes.c_int64 * len(counts))(*counts)
+        ticket = self.lib.hvd_adapter_allreduce_async(self.h, _ptrs(tensors), _ptrs(outputs), cnt, len(counts), dtype,
+                                                      -1, prescale, postscale, _ptrs(list(peers)), len(peers), err, 512)
+        assert ticket >= 0, err.value.decode()
+        return ticket
+
+    def wait_all(self):
+        err = ctypes.create_string_buffer(512)
+        rc = self.lib.hvd_adapter_wait_all(self.h, err, 512)
+        return rc, err.value.decode()
+
+    def op_times(self, ticket):
+        q, r, c = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+        assert self.lib.hvd_adapter_op_times(self.h, ticket, ctypes.byref(q), ctypes.byref(r), ctypes.byref(c)) == 0
+        return q.value, r.value, c.value
 
     def allreduce(self, tensors, outputs, counts, dtype, prescale, postscale, peers=()):
         err = ctypes.create_string_buffer(512)
@@ -359,5 +387,89 @@ def test_adasum_dispatch_hooks(gpu, orc, adapter):
         want = orc.adasum_scaled_add(a, b, 0.75, 1.25, F32)
         got = gpu.download(d_a, np.float32)
         assert np.all(np.abs(got - want) <= np.spacing(np.abs(want)))
+    finally:
+        h.close()
+
+
+def test_two_consecutive_executes_on_alternating_slots_are_both_in_flight(gpu, orc, adapter):
+    """GPUOpContext::FinalizeGPUQueue hands the wait to a finalizer thread and returns
+    (ops/gpu_operations.cc:50-99), so the second Execute is launched on the other stream slot while
+    the first response still runs: both calls return before either response completes.  Each
+    response is 8 x 32 MiB of float32 with four peers (several hundred microseconds of kernels
+    against tens of microseconds of host time per Execute)."""
+    import torch
+    n_entries, count = 8, 8 << 20
+    g = torch.Generator(device="cuda")
+    g.manual_seed(11)
+    sets = []
+    for _ in range(2):
+        src = torch.randn(n_entries * count, generator=g, device="cuda", dtype=torch.float32)
+        dst = torch.zeros(n_entries * count, device="cuda", dtype=torch.float32)
+        sets.append((src, dst))
+    peer = torch.randn(n_entries * count, generator=g, device="cuda", dtype=torch.float32)
+    torch.cuda.synchronize()
+    h = Harness(adapter, gpu, num_streams=2, fb_bytes=n_entries * count * 4 + 4096)
+    try:
+        def args(k):
+            src, dst = sets[k]
+            return ([src.data_ptr() + 4 * count * i for i in range(n_entries)],
+                    [dst.data_ptr() + 4 * count * i for i in range(n_entries)], [count] * n_entries)
+        # warm-up: plans, streams and event pools exist afterwards
+        for k in range(2):
+            h.allreduce_async(*args(k), F32, 0.5, 1.0, [peer.data_ptr()] * 4)
+        rc, msg = h.wait_all()
+        assert rc == 0, msg
+        torch.cuda.synchronize()
+        first = h.allreduce_async(*args(0), F32, 0.5, 2.0, [peer.data_ptr()] * 4)
+        second = h.allreduce_async(*args(1), F32, 0.5, 2.0, [peer.data_ptr()] * 4)
+        done_when_both_were_queued = adapter.hvd_adapter_completed(h.h) - 2
+        rc, msg = h.wait_all()
+        assert rc == 0, msg
+        t1, t2 = h.op_times(first), h.op_times(second)
+        assert done_when_both_were_queued == 0
+        assert t2[1] < t1[2] and t2[1] < t2[2], (t1, t2)   # the second Execute returned before either completed
+        assert t1[1] <= t2[0]                                # and was called after the first had returned
+        assert h.state()[0] == 0                             # four responses: the slot rotated back
+        # the callbacks ran after the results were there
+        for k in range(2):
+            src, dst = sets[k]
+            x = src[:4096].cpu().numpy()
+            w = orc.scale_buffer(x, 0.5, F32)
+            p = peer[:4096].cpu().numpy()
+            for _ in range(4):
+                w = orc.sum(p, w, F32)
+            w = orc.scale_buffer(w, 2.0, F32)
+            assert np.array_equal(dst[:4096].cpu().numpy().view(np.uint32), w.view(np.uint32))
+        print("Execute returned after %.0f / %.0f us; responses completed %.0f / %.0f us after the first call"
+              % ((t1[1] - t1[0]) * 1e6, (t2[1] - t2[0]) * 1e6, (t1[2] - t1[0]) * 1e6, (t2[2] - t1[0]) * 1e6))
+    finally:
+        h.close()
+
+
+@pytest.mark.parametrize("threads", [0, 1, 2])
+def test_a_run_of_responses_with_and_without_finalizer_threads(gpu, orc, adapter, threads):
+    """20 fused responses queued back to back over two slots; with no finalizer thread every
+    completion runs on the calling thread (Execute then returns after the response has finished)."""
+    rng = np.random.default_rng(12)
+    counts = [5, 1000, 3, 70001, 256, 1]
+    total = sum(counts)
+    reps = 20
+    v = rng.standard_normal(reps * total).astype(np.float32)
+    d_v, d_o = gpu.upload(v), gpu.empty(v.nbytes, fill=0)
+    offs = np.concatenate([[0], np.cumsum(counts)])
+    h = Harness(adapter, gpu, num_streams=2, finalizer_threads=threads)
+    try:
+        tickets = []
+        for r in range(reps):
+            t = [d_v.data_ptr() + 4 * (r * total + int(o)) for o in offs[:-1]]
+            o = [d_o.data_ptr() + 4 * (r * total + int(o)) for o in offs[:-1]]
+            tickets.append(h.allreduce_async(t, o, counts, F32, 0.25, 1.0))
+            if threads == 0:
+                assert adapter.hvd_adapter_completed(h.h) == r + 1
+        rc, msg = h.wait_all()
+        assert rc == 0, msg
+        assert adapter.hvd_adapter_completed(h.h) == reps
+        got = gpu.download(d_o, np.float32)
+        assert np.array_equal(got, orc.scale_buffer(v, 0.25, F32))
     finally:
         h.close()
