@@ -10,19 +10,29 @@ the collective replaced by the local sum.  One "step" is REPS passes of that pip
 tensor sets that rotate so that no pass finds its inputs in the 256 MB Infinity Cache.  Inputs
 are resident in HBM before the timed region starts; everything runs on one stream.
 
-Prints ONE JSON line.  `value` is ALGORITHMIC GB/s of the whole step (pack = P_in + P_buf,
-reduce = (k+2) C, unpack = P_buf + P_out; the bytes a pipeline must move with the fusion buffer
-materialised on both sides of the collective) -- not an HBM counter: inside a cycle the fusion
-buffer is handed from kernel to kernel through the Infinity Cache, so a pipeline's algorithmic
-rate can exceed what any one of its kernels streams out of HBM.  The HBM claim is `roofline`:
-the dominant kernel of the workload launched back to back on rotating buffers, algorithmic bytes
-per launch over its average duration from HIP events on its stream, against the 8 TB/s peak.
-`cpu_baseline` is the CPU oracle (a restatement of the reference's CPU path) on one host core
-over the same workload.  `extra` carries the other configurations, each with the same roofline
-block for every kernel family it launches (`kernels`), the dominant one repeated as `roofline`.
+Prints ONE JSON line on stdout, small enough for a reader who keeps the last 8 KB: the contract's keys
+in full, every other configuration as one row per pipeline and one row per kernel loop.  The same
+results with the description of what each figure timed go to stderr as one line that begins with
+"DETAIL ".  `value` is ALGORITHMIC GB/s of the whole step (pack = P_in + P_buf, reduce = (k+2) C,
+unpack = P_buf + P_out; the bytes a pipeline must move with the fusion buffer materialised on both
+sides of the collective) -- not an HBM counter: inside a cycle the fusion buffer is handed from
+kernel to kernel through the Infinity Cache, so a pipeline's algorithmic rate can exceed what any
+one of its kernels streams out of HBM (`value_kind` says so; `hbm_GB/s` is the counter-derived HBM
+rate of the roofline kernel).  `ms_per_step` is the wall-clock mean of the K timed steps;
+`ms_per_step_median_min_max` comes from a HIP event pair around each step on the pipeline's stream.
+The HBM claim is `roofline`: the dominant kernel of the workload launched back to back on rotating
+buffers, algorithmic bytes per launch over its launch time from HIP events on its stream (mean over
+ten batches of launches, with median / min / max of the batches), against the 8 TB/s peak.
+`cpu_baseline` is the CPU oracle (a restatement of the reference's CPU path) on one host core over
+the same workload.  `extra` carries the other configurations: C1-C5 pipelines on one and two
+streams, C1 and C5 once more through the C++ adapter's GPUAllreduce::Execute with its finalizer
+threads, the allgather buffer's copies, the device's own 1 GiB copy rates, and one row per kernel
+loop (an unpack's `in_pipeline_us` is its time right behind the reduce-sum that wrote its buffer).
 
 `--kernel-only <config>` runs exactly the back-to-back kernel loops of one configuration and
-nothing else, for rocprofv3 (the summaries under profiles/ come from these runs).
+nothing else, for rocprofv3 (the summaries under profiles/ come from these runs); `--calibrate`
+launches two plain 256 MiB copies that are not the library's kernels, whose known byte counts scale
+the profiler's FETCH_SIZE and WRITE_SIZE counters.
 """
 import argparse
 import json
@@ -46,28 +56,45 @@ REPS = 50
 ROTATE = 6
 
 # HBM bytes per launch, per kernel of the --kernel-only loops, from rocprofv3 FETCH_SIZE and
-# WRITE_SIZE runs (KiB per dispatch), each scaled by what the same counter reads for a plain
-# 256 MiB device copy (`bench.py --calibrate`).  The summaries with the commands are the files
-# named here under profiles/; tests/test_host_logic.py re-derives every figure from them.
+# WRITE_SIZE runs (KiB per dispatch), each scaled by what the same counter reads for two plain
+# 256 MiB device copies of known size that are not the library's own kernels
+# (`bench.py --calibrate`).  The summaries with the commands are the files named here under
+# profiles/; tests/test_host_logic.py re-derives every figure from them.
 TRAFFIC_BYTES_MEASURED = {
-    "c1.pack": 125571679,
-    "c1.reduce": 184760472,
-    "c1.unpack": 125579671,
-    "c2.pack": 93208463,
-    "c2.unpack": 92594017,
-    "c3.pack": 194421549,
-    "c3.reduce": 71756749,
-    "c3.unpack": 197818970,
-    "c4.combine": 662273259,
-    "c4h.combine": 331102123,
-    "c5.pack": 123465051,
-    "c5.reduce": 181653632,
-    "c5.reduce_single": 475145891,
-    "c5.scale_single": 318055645,
-    "c5.unpack": 123473213,
-    "copy.library": 2155922559,
-    "copy.runtime": 2123025630,
-    "copy.torch": 2123026410,
+    "ag.pack": 138114590,
+    "ag.pack_small": 12592637,
+    "ag.unpack": 1097092646,
+    "ag.unpack_small": 99870512,
+    "c1.pack": 126061635,
+    "c1.reduce": 187599846,
+    "c1.reduce+unpack": 313695480,
+    "c1.unpack": 126064739,
+    "c2.pack": 93545928,
+    "c2.unpack": 92914168,
+    "c3.pack": 196388983,
+    "c3.reduce": 73234670,
+    "c3.reduce_8MiB_apart": 73234321,
+    "c3.unpack": 197367728,
+    "c3.unpack_postscale4": 197377999,
+    "c4.combine": 674534013,
+    "c4h.combine": 337233779,
+    "c5.pack": 123955198,
+    "c5.reduce": 184445164,
+    "c5.reduce+unpack": 308444908,
+    "c5.reduce_single": 482447512,
+    "c5.scale_single": 321693411,
+    "c5.unpack": 123952383,
+    "copy.library": 2164248147,
+    "copy.runtime": 2147401707,
+    "copy.torch": 2147400909,
+}
+# Kernel-trace duration (ns) of an unpack launched right behind the reduce-sum that wrote its buffer (the
+# `<config>.reduce+unpack` loops), from the same summaries: what the unpack takes in a cycle, where its
+# input comes out of the Infinity Cache.  HIP events cannot single it out without getting between the two
+# kernels, so the figure is carried from the profile and pinned by the same test.
+IN_PIPELINE_NS_MEASURED = {
+    "c1.unpack": 18108.5,
+    "c5.unpack": 18059.2,
 }
 TRAFFIC_PROFILE = {
     "c1": "profiles/c1_resnet50_fp32_kernels.txt",
@@ -76,10 +103,11 @@ TRAFFIC_PROFILE = {
     "c4": "profiles/c4_adasum_fp32_kernels.txt",
     "c5": "profiles/c5_gpt2_xl_fp16_kernels.txt",
     "copy": "profiles/device_copy_1GiB_three_ways.txt",
+    "ag": "profiles/ag_allgather_kernels.txt",
 }
 
 CONFIGS = ("c1", "c2", "c3", "c4", "c5")
-KERNEL_ONLY = CONFIGS + ("c4h", "copy")
+KERNEL_ONLY = CONFIGS + ("c4h", "copy", "ag")
 
 
 def parse():
@@ -94,7 +122,8 @@ def parse():
                     help="only the back-to-back kernel loops of one configuration (for rocprofv3 runs): c1 ResNet-50 "
                          "fp32 cycle, c2 fusion stress, c3 BERT-large fp32->fp16 cycle with 7 peers on the 1/8 share, "
                          "c4 Adasum 2 x 2^25 fp32, c4h the same in fp16, c5 GPT-2 XL fp16 cycle and embedding, copy 1 GiB moved by the "
-                         "library's kernel, by hipMemcpyAsync and by an elementwise kernel of torch; "
+                         "library's kernel, by hipMemcpyAsync and by an elementwise kernel of torch, ag the allgather "
+                         "fusion buffer's pack and unpack (8 ranks x 128 entries) at a 6 MB and at a 66 MB slab; "
                          "--steps launches per kernel after --warmup")
     ap.add_argument("--calibrate", action="store_true",
                     help="only launch a plain 256 MiB device copy (scales rocprofv3 byte counters)")
@@ -105,35 +134,85 @@ def parse():
 # timing
 # ----------------------------------------------------------------------------------------------
 
-def timed(fn, sync, steps, warmup):
-    """Wall time of `steps` calls of fn bracketed by synchronisation on both sides."""
+def timed(fn, sync, steps, warmup, stream=None):
+    """Wall time of `steps` calls of fn bracketed by synchronisation on both sides.  With `stream`
+    (everything fn queues goes onto that one stream) every call is bracketed by a HIP event pair on
+    it as well, and the per-call stream times come back as a second value: (seconds per call,
+    [seconds of each call] or None)."""
+    import torch
+    from horovod_amd import Timer
+    for _ in range(warmup):
+        fn()
+    sync()
+    torch.cuda.synchronize()
+    timers = [Timer() for _ in range(steps)] if stream is not None else []
+    t0 = time.perf_counter()
+    for i in range(steps):
+        if timers:
+            timers[i].start(stream)
+        fn()
+        if timers:
+            timers[i].stop(stream)
+    sync()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / steps
+    each = [t.elapsed_ms() * 1e-3 for t in timers] or None
+    for t in timers:
+        t.destroy()
+    return sec, each
+
+
+def spread(values, scale=1.0, digits=4):
+    """[median, min, max] of a list of times."""
+    v = sorted(values)
+    n = len(v)
+    med = v[n // 2] if n % 2 else 0.5 * (v[n // 2 - 1] + v[n // 2])
+    return [round(med * scale, digits), round(v[0] * scale, digits), round(v[-1] * scale, digits)]
+
+
+def event_timed(fn, stream, steps, warmup, batches=10):
+    """Stream time per call of fn from HIP events recorded on `stream`: the launches go out in
+    `batches` runs, each bracketed by an event pair (an event per launch would put its own
+    2-3 us between the kernels).  Returns (mean seconds per call over all batches,
+    [mean seconds per call of each batch])."""
+    from horovod_amd import Timer
+    for _ in range(warmup):
+        fn()
+    stream.synchronize()
+    batches = max(1, min(batches, steps))
+    per = max(1, steps // batches)
+    timers = [Timer() for _ in range(batches)]
+    for t in timers:
+        t.start(stream)
+        for _ in range(per):
+            fn()
+        t.stop(stream)
+    each = [t.elapsed_ms() * 1e-3 / per for t in timers]
+    for t in timers:
+        t.destroy()
+    return sum(each) / len(each), each
+
+
+def timed_batches(fn, sync, steps, warmup, batches=5):
+    """Wall time per call of fn over `batches` runs, each bracketed by synchronisation (for pipelines
+    that spread over two streams, where no single stream's events bracket a call).  Returns (mean
+    seconds per call, [mean seconds per call of each batch])."""
     import torch
     for _ in range(warmup):
         fn()
     sync()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        fn()
-    sync()
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) / steps
-
-
-def event_timed(fn, stream, steps, warmup):
-    """Average stream time per call of fn, from HIP events recorded on `stream`."""
-    from horovod_amd import Timer
-    for _ in range(warmup):
-        fn()
-    stream.synchronize()
-    t = Timer()
-    t.start(stream)
-    for _ in range(steps):
-        fn()
-    t.stop(stream)
-    ms = t.elapsed_ms()
-    t.destroy()
-    return ms / steps * 1e-3
+    batches = max(1, min(batches, steps))
+    per = max(1, steps // batches)
+    each = []
+    for _ in range(batches):
+        t0 = time.perf_counter()
+        for _ in range(per):
+            fn()
+        sync()
+        torch.cuda.synchronize()
+        each.append((time.perf_counter() - t0) / per)
+    return sum(each) / len(each), each
 
 
 _PAIR = []
@@ -204,16 +283,21 @@ class Case:
     """One kernel at one grid.  fn() queues one launch on `stream` (the next rotating buffer set
     every call); alg = algorithmic bytes per launch; kernel = its name as a profiler prints it
     (template arguments: ..., 0 pack / 1 unpack, 0 non-temporal / 1 write-through stores).
-    parts: for a call that launches several kernels, [(kernel, algorithmic bytes)] per kernel."""
+    parts: for a call that launches several kernels, [(kernel, algorithmic bytes, algorithmic bytes read)] per
+    kernel; reads: the algorithmic bytes read of a single-kernel call when that is not half of alg."""
 
-    def __init__(self, key, kernel, fn, alg, what, workgroups=None, cleanup=None, parts=None):
+    def __init__(self, key, kernel, fn, alg, what, workgroups=None, cleanup=None, parts=None, follows=None, reads=None):
         self.key, self.kernel, self.fn, self.alg, self.what, self.workgroups = key, kernel, fn, alg, what, workgroups
         self.cleanup = cleanup  # destroys the plans behind fn (the closures hold the device memory)
-        self.parts = parts or [(kernel, alg)]
+        # per kernel of the call: (name, algorithmic bytes, of which read); a copy reads half of what it moves
+        self.parts = parts or [(kernel, alg, alg // 2 if reads is None else reads)]
+        # (case of the first kernel alone, case of the second kernel alone) when fn launches the two back to
+        # back on the same buffer, so that the second finds its input in the Infinity Cache (informative)
+        self.follows = follows
 
 
 def cycle_cases(cfg, counts, tdtype, bdtype, std, peers, share_world, stream, pack_kernel, reduce_kernel,
-                unpack_kernel, seed0):
+                unpack_kernel, seed0, extra_postscale=None, pack_rotating=False):
     """Pack, reduce-sum and unpack of ONE fusion cycle, each launched back to back:
     pack reads another replica's tensors every launch and writes the slot's one fusion buffer (as the
     reference keeps one per stream slot); the reduce-sum and the unpack rotate over ROTATE buffers."""
@@ -258,12 +342,27 @@ def cycle_cases(cfg, counts, tdtype, bdtype, std, peers, share_world, stream, pa
     def pack():
         sets[rot()][2].pack(fb_pack.data_ptr(), 0.125, stream)
 
+    def pack_rotating_destination():
+        i = rot()
+        sets[i][2].pack(fbs[i].data_ptr(), 0.125, stream)
+
     def reduce():
         i = rot()
         H.reduce_sum_k(fbs[i].data_ptr(), [p.data_ptr() for p in peer_bufs[i]], share, bdtype, stream)
 
     def unpack():
         i = rot()
+        sets[i][2].unpack(fbs[i].data_ptr(), 1.0, stream)
+
+    def unpack_scaled():
+        i = rot()
+        sets[i][2].unpack(fbs[i].data_ptr(), extra_postscale, stream)
+
+    def reduce_then_unpack():
+        # the drop-in's order: the collective has just written the buffer (through the Infinity Cache)
+        # when the unpack reads it
+        i = rot()
+        H.reduce_sum_k(fbs[i].data_ptr(), [p.data_ptr() for p in peer_bufs[i]], share, bdtype, stream)
         sets[i][2].unpack(fbs[i].data_ptr(), 1.0, stream)
 
     def cleanup():
@@ -275,13 +374,47 @@ def cycle_cases(cfg, counts, tdtype, bdtype, std, peers, share_world, stream, pa
         Case(cfg + ".pack", pack_kernel, pack, payload * (ts + bs),
              "pack with prescale 0.125 of %d tensors (%d payload bytes in, %d in the buffer); tensors of another replica "
              "every launch, the slot's one fusion buffer as destination" % (len(counts), payload * ts, payload * bs),
-             plan0.num_chunks, cleanup),
+             plan0.num_chunks, cleanup, reads=payload * ts),
         Case(cfg + ".reduce", reduce_kernel, reduce, (peers + 2) * share * bs,
              "resident chunk of %d bytes += %d peer chunk(s) in one pass; %d (resident, peers) sets rotated"
-             % (share * bs, peers, ROTATE), (share + tile - 1) // tile),
+             % (share * bs, peers, ROTATE), (share + tile - 1) // tile, reads=(peers + 1) * share * bs),
         Case(cfg + ".unpack", unpack_kernel, unpack, payload * (bs + ts),
-             "unpack (postscale 1.0) of the same tensors; fusion buffer and outputs of another replica every launch"),
+             "unpack (postscale 1.0) of the same tensors; fusion buffer and outputs of another replica every launch",
+             plan0.num_chunks, reads=payload * bs),
     ]
+    if pack_rotating:
+        cases.append(Case(cfg + ".pack_rotating_destination", pack_kernel, pack_rotating_destination, payload * (ts + bs),
+                          "the same pack into a different fusion buffer every launch (%d rotated): what the pack takes when "
+                          "its destination, like the unpack's, is not resident in the Infinity Cache" % ROTATE,
+                          plan0.num_chunks, reads=payload * ts))
+    if extra_postscale is not None:
+        cases.append(Case(cfg + ".unpack_postscale%g" % extra_postscale, unpack_kernel, unpack_scaled, payload * (bs + ts),
+                          "the same unpack with postscale %g" % extra_postscale, plan0.num_chunks, reads=payload * bs))
+    if share_world == 1:
+        cases.append(Case(cfg + ".reduce+unpack", reduce_kernel + " + " + unpack_kernel, reduce_then_unpack,
+                          (peers + 2) * share * bs + payload * (bs + ts),
+                          "the reduce-sum and, right behind it on the same buffer, the unpack: the unpack's input comes "
+                          "out of the Infinity Cache as in a cycle (a kernel trace gives each kernel's own duration)",
+                          None, None, [(reduce_kernel, (peers + 2) * share * bs, (peers + 1) * share * bs),
+                                       (unpack_kernel, payload * (bs + ts), payload * bs)],
+                          follows=(cfg + ".reduce", cfg + ".unpack")))
+    if peers >= 3:
+        # The worst placement of a staging ring: the resident chunk and its peers exactly 8 MiB apart
+        # (a 1/8 share of a 64 MiB buffer is 8 MiB), against the back-to-back placement above.
+        gap = 8 << 20
+        assert share * bs <= gap
+        ring = randn_bytes(ROTATE * (peers + 1) * gap, bt, std, seed0 + 60)
+        torch.cuda.synchronize()
+
+        def reduce_pow2():
+            i = rot()
+            at = ring.data_ptr() + i * (peers + 1) * gap
+            H.reduce_sum_k(at, [at + (p + 1) * gap for p in range(peers)], share, bdtype, stream)
+
+        cases.append(Case(cfg + ".reduce_8MiB_apart", reduce_kernel, reduce_pow2, (peers + 2) * share * bs,
+                          "the same sum with the resident chunk and the %d peer chunks exactly 8 MiB apart in one "
+                          "allocation (the spacing of a power-of-two staging ring)" % peers, (share + tile - 1) // tile,
+                          reads=(peers + 1) * share * bs))
     return cases
 
 
@@ -296,7 +429,7 @@ def build_cases(cfg):
         g0 = W.fuse([4 * c for c in counts])[0]
         return cycle_cases("c1", [counts[i] for i in g0], F32, F32, 1e-3, 1, 1, s,
                            "xfer_k<Scale<float, float>, 0, 1>", "reduce_k<float, 1, 1>",
-                           "xfer_k<Copy<unsigned int>, 1, 0>", 1000)
+                           "xfer_k<Copy<unsigned int>, 1, 0>", 1000, pack_rotating=True)
     if cfg == "c2":
         counts = W.stress_counts(seed=3)
         cases = cycle_cases("c2", counts, F32, F32, 1.0, 1, 1, s, "xfer_k<Scale<float, float>, 0, 1>",
@@ -307,7 +440,7 @@ def build_cases(cfg):
         g1 = W.fuse([2 * c for c in counts])[1]
         return cycle_cases("c3", [counts[i] for i in g1], F32, F16, 1e-4, 7, 8, s,
                            "xfer_k<PackF32F16, 0, 1>", "reduce_k<_Float16, 7, 1>",
-                           "xfer_k<UnpackF16F32, 1, 0>", 3000)
+                           "xfer_k<UnpackF16F32, 1, 0>", 3000, extra_postscale=4.0)
     if cfg == "c5":
         counts = [W.numel(x) for x in W.gpt2_xl_shapes()]
         groups = W.fuse([2 * c for c in counts])
@@ -336,7 +469,7 @@ def build_cases(cfg):
                  "the embedding (%d halves) scaled by 0.125 from tensor to output; 3 pairs rotated" % n,
                  (2 * n + 4095) // 4096),
             Case("c5.reduce_single", "reduce_k<_Float16, 1, 1>", reduce_emb, 6 * n,
-                 "the embedding summed in place with one peer; 3 pairs rotated", (2 * n + 4095) // 4096),
+                 "the embedding summed in place with one peer; 3 pairs rotated", (2 * n + 4095) // 4096, reads=4 * n),
         ]
         return cases
     if cfg in ("c4", "c4h"):
@@ -366,7 +499,9 @@ def build_cases(cfg):
         return [Case(cfg + ".combine", k1 + " + " + k2, combine, 5 * n * es,
                      "Adasum combine of two vectors of 2^25 elements in 64 layers: first pass 2 N s bytes (leaves what "
                      "pays in the Infinity Cache), second pass 3 N s bytes; 4 pairs rotated", None, plan.destroy,
-                     parts=[(k1, 2 * n * es), (k2, 3 * n * es)])]
+                     parts=[(k1, 2 * n * es, 2 * n * es), (k2, 3 * n * es, 2 * n * es)])]
+    if cfg == "ag":
+        return allgather_cases(s)
     if cfg == "copy":
         # One GiB copied to another by the library's copy kernel, by the runtime's own device-to-device
         # hipMemcpyAsync and by an elementwise kernel of torch: what this device streams, whoever asks.
@@ -416,12 +551,19 @@ def measure_cases(cases, steps=100, warmup=10):
     s = stream_pair()[0]
     out = []
     for c in cases:
-        sec = event_timed(c.fn, s, steps, warmup)
+        sec, each = event_timed(c.fn, s, steps, warmup)
         gbs = c.alg / sec / 1e9
         out.append({"bound": "hbm", "kernel": c.kernel, "case": c.key, "launch_us": round(sec * 1e6, 2),
+                    "launch_us_median_min_max": spread(each, 1e6, 2), "timed_batches": len(each),
                     "algorithmic_bytes_per_launch": c.alg, "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                     "traffic": TRAFFIC_BYTES_MEASURED.get(c.key), "workgroups": c.workgroups, "timed": c.what})
+    for b in out:
+        ns = IN_PIPELINE_NS_MEASURED.get(b["case"])
+        if ns:
+            b["in_pipeline_us"] = round(ns / 1e3, 2)
+            b["in_pipeline_frac"] = round(b["algorithmic_bytes_per_launch"] / ns / HBM_PEAK_GBS, 4)
+            b["in_pipeline_from"] = "kernel-trace duration behind the reduce-sum that wrote its buffer (%s.reduce+unpack in the profile)" % b["case"].split(".")[0]
     return out
 
 
@@ -445,8 +587,9 @@ class PipelineRun:
     the same stream(s) and share the one fusion buffer of each stream slot."""
 
     def __init__(self, shapes, tdtype, bdtype, std, peers, fraction, streams, replicas, arrays=False,
-                 completion_events=None, record_with_unpack=False):
+                 completion_events=None, record_with_unpack=False, postscale=1.0):
         import torch
+        self.postscale = postscale
         from horovod_amd import dtype_size, workloads as W
         from horovod_amd.pipeline import AllreducePipeline
         es = dtype_size(tdtype)
@@ -477,7 +620,7 @@ class PipelineRun:
         _, _, pipe, peer_bufs = self.reps[self.turn % len(self.reps)]
         # a single-cycle configuration alternates its passes over the stream slots
         first_slot = self.turn if len(pipe.cycles) == 1 else 0
-        pipe.run(0.125, 1.0, (lambda ci, p: peer_bufs[p].data_ptr()) if self.peers else None, self.peers,
+        pipe.run(0.125, self.postscale, (lambda ci, p: peer_bufs[p].data_ptr()) if self.peers else None, self.peers,
                  self.fraction, True, first_slot=first_slot)
 
     def sync(self):
@@ -492,6 +635,90 @@ class PipelineRun:
         for _, _, pipe, _ in self.reps:
             pipe.destroy()
         self.reps = []
+        torch.cuda.empty_cache()
+
+
+class AdapterRun:
+    """The same pipelines through the C++ adapter: every fused response goes through
+    GPUAllreduce::Execute (pack -> sum with the peer buffer -> unpack with the completion event bound to
+    it -> FinalizeGPUQueue), which returns once the kernels are queued; finalizer threads, one per
+    stream slot, wait for the events and call the entries' callbacks, and the stream slot rotates after
+    every response (ops/gpu_operations.cc:50-103).  The calling thread plays Horovod's background thread."""
+
+    def __init__(self, shapes, dtype, std, slots, replicas):
+        import ctypes
+        import torch
+        from horovod_amd import dtype_size, workloads as W
+        from horovod_amd._lib import adapter_lib
+        lib = adapter_lib()
+        VP = ctypes.c_void_p
+        lib.hvd_adapter_create_ex.restype = VP
+        lib.hvd_adapter_create_ex.argtypes = [ctypes.c_int] * 4 + [VP, ctypes.c_int]
+        lib.hvd_adapter_destroy.argtypes = [VP]
+        lib.hvd_adapter_prepare.argtypes = [VP, VP, VP, VP, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        lib.hvd_adapter_execute_prepared.argtypes = [VP, ctypes.c_int, ctypes.c_double, ctypes.c_double, VP, ctypes.c_int,
+                                                     ctypes.c_char_p, ctypes.c_size_t]
+        lib.hvd_adapter_wait_all.argtypes = [VP, ctypes.c_char_p, ctypes.c_size_t]
+        lib.hvd_adapter_reset_tickets.argtypes = [VP]
+        self.lib = lib
+        es = dtype_size(dtype)
+        self.es = es
+        self.counts = [W.numel(x) for x in shapes]
+        groups = W.fuse([c * es for c in self.counts])
+        self.groups = groups
+        need = max([sum((self.counts[i] * es + 15) // 16 * 16 for i in g) for g in groups if len(g) > 1] + [16]) + 4096 * es
+        self.fbs = [zeros_bytes(need) for _ in range(slots)]
+        self.h = lib.hvd_adapter_create_ex(slots, 1, 0, 0, (VP * slots)(*[b.data_ptr() for b in self.fbs]), slots)
+        # the run's one pair of streams, created before any other (see stream_pair)
+        lib.hvd_adapter_use_streams.argtypes = [VP, VP]
+        lib.hvd_adapter_use_streams(self.h, (VP * slots)(*[st.handle.value for st in stream_pair()[:slots]]))
+        self.err = ctypes.create_string_buffer(512)
+        self.reps = []
+        for r in range(replicas):
+            src = DeviceSet(self.counts, es, lambda n: randn_bytes(n, torch_dtype(dtype), std, 1 + r))
+            dst = DeviceSet(self.counts, es, zeros_bytes)
+            # one peer buffer, sized for the largest response, serves every response of the replica
+            largest = max(sum((self.counts[i] * es + 15) // 16 * 16 for i in g) for g in groups)
+            peer = randn_bytes((largest + 255) // 256 * 256, torch_dtype(dtype), std, 100 + 16 * r)
+            ids = []
+            for g in groups:
+                n = len(g)
+                ids.append(lib.hvd_adapter_prepare(self.h, (VP * n)(*[src.ptrs[i] for i in g]),
+                                                   (VP * n)(*[dst.ptrs[i] for i in g]),
+                                                   (ctypes.c_int64 * n)(*[self.counts[i] for i in g]), n, dtype, -1))
+            self.reps.append((src, dst, peer, ids, (VP * 1)(peer.data_ptr())))
+        torch.cuda.synchronize()
+        self.turn = 0
+
+    def one_pass(self):
+        self.turn += 1
+        _, _, _, ids, peers = self.reps[self.turn % len(self.reps)]
+        for i in ids:
+            if self.lib.hvd_adapter_execute_prepared(self.h, i, 0.125, 1.0, peers, 1, self.err, 512) < 0:
+                raise RuntimeError(self.err.value.decode())
+
+    def sync(self):
+        if self.lib.hvd_adapter_wait_all(self.h, self.err, 512) != 0:
+            raise RuntimeError(self.err.value.decode())
+        self.lib.hvd_adapter_reset_tickets(self.h)
+
+    def algorithmic_bytes(self):
+        # fused: pack 2P + reduce 3C (C = the padded buffer) + unpack 2P; single entry: scale 2P + reduce 3P
+        total = 0
+        for g in self.groups:
+            payload = sum(self.counts[i] for i in g) * self.es
+            if len(g) > 1:
+                total += 4 * payload + 3 * sum((self.counts[i] * self.es + 15) // 16 * 16 for i in g)
+            else:
+                total += 5 * payload
+        return total
+
+    def destroy(self):
+        import torch
+        self.sync()
+        self.lib.hvd_adapter_destroy(self.h)
+        self.reps = []
+        self.fbs = []
         torch.cuda.empty_cache()
 
 
@@ -724,57 +951,88 @@ def per_tensor_comparator(reps=20):
     return out
 
 
-def allgather_extra(steps):
-    """Allgather fusion buffer (ops/collective_operations.cc:234-288): 8 ranks, 128 entries per rank with
-    the stress workload's size mix.  This GPU packs its own slab at its displacement (the other slabs
-    arrive by the collective, which is not built) and unpacks one component per (entry, rank).  Each
-    direction is one batched copy through the descriptor-array entry point; 4 independent sets rotate."""
+def allgather_cases(s):
+    """Allgather fusion buffer (ops/collective_operations.cc:234-288, GPU copies ops/gpu_operations.cc:350-363):
+    8 ranks, 128 entries per rank.  This GPU packs its own slab at its displacement (the other slabs arrive
+    by the collective, which is not built) and unpacks one component per (entry, rank): 1,024 copies.  Each
+    direction is one batched copy through the descriptor-array entry point.  Two sizes: the stress
+    workload's size mix as it is (a 6 MB slab: the pack is a launch floor) and eleven times that (a 66 MB
+    slab, a 528 MB buffer: bandwidth-bound)."""
     import ctypes
     import torch
     import horovod_amd
     from horovod_amd import workloads as W
-    s = stream_pair()[0]
     world, es = 8, 4
-    counts = W.stress_counts(seed=21, n=128)
-    slab = es * sum(counts)
-    sets = []
-    for r in range(4):
-        src = DeviceSet(counts, es, lambda n: randn_bytes(n, torch.float32, 1.0, 60 + r))
-        fusion = torch.empty(world * slab, dtype=torch.uint8, device="cuda")
-        outs = [torch.empty(world * c * es, dtype=torch.uint8, device="cuda") for c in counts]
-        pack_dst, at = [], 3 * slab  # this rank's displacement (rank 3 of 8)
-        for c in counts:
-            pack_dst.append(fusion.data_ptr() + at)
-            at += c * es
-        un_dst, un_src, un_sz = [], [], []
-        for rank in range(world):
-            at = rank * slab
-            for i, c in enumerate(counts):
-                un_dst.append(outs[i].data_ptr() + rank * c * es)
-                un_src.append(fusion.data_ptr() + at)
-                un_sz.append(c * es)
-                at += c * es
-        # the descriptor arrays as the C caller holds them, built once
-        VP, SZ = ctypes.c_void_p, ctypes.c_size_t
-        pack_args = ((VP * len(counts))(*pack_dst), (VP * len(counts))(*src.ptrs),
-                     (SZ * len(counts))(*[c * es for c in counts]), len(counts))
-        un_args = ((VP * len(un_dst))(*un_dst), (VP * len(un_dst))(*un_src), (SZ * len(un_dst))(*un_sz), len(un_dst))
-        sets.append((src, fusion, outs, pack_args, un_args))
-    torch.cuda.synchronize()
     copy = horovod_amd.lib().hvdhip_batched_d2d_memcpy
-    turn = [0]
+    cases = []
+    for tag, mult, rotate in (("_small", 1, 4), ("", 11, 3)):
+        counts = [c * mult for c in W.stress_counts(seed=21, n=128)]
+        slab = es * sum(counts)
+        sets = []
+        for r in range(rotate):
+            src = DeviceSet(counts, es, lambda n: randn_bytes(n, torch.float32, 1.0, 60 + r))
+            fusion = randn_bytes(world * slab, torch.float32, 1.0, 70 + r)
+            out_set = DeviceSet([world * c for c in counts], es, zeros_bytes)
+            pack_dst, at = [], 3 * slab  # this rank's displacement (rank 3 of 8)
+            for c in counts:
+                pack_dst.append(fusion.data_ptr() + at)
+                at += c * es
+            un_dst, un_src, un_sz = [], [], []
+            for rank in range(world):
+                at = rank * slab
+                for i, c in enumerate(counts):
+                    un_dst.append(out_set.ptrs[i] + rank * c * es)
+                    un_src.append(fusion.data_ptr() + at)
+                    un_sz.append(c * es)
+                    at += c * es
+            # the descriptor arrays as the C caller holds them, built once
+            VP, SZ = ctypes.c_void_p, ctypes.c_size_t
+            pack_args = ((VP * len(counts))(*pack_dst), (VP * len(counts))(*src.ptrs),
+                         (SZ * len(counts))(*[c * es for c in counts]), len(counts))
+            un_args = ((VP * len(un_dst))(*un_dst), (VP * len(un_dst))(*un_src), (SZ * len(un_dst))(*un_sz), len(un_dst))
+            sets.append((src, fusion, out_set, pack_args, un_args))
+        torch.cuda.synchronize()
+        turn = [0]
 
-    def gather_step():
-        i = turn[0] = (turn[0] + 1) % len(sets)
-        horovod_amd.check(copy(*sets[i][3], s.handle), "hvdhip_batched_d2d_memcpy")
-        horovod_amd.check(copy(*sets[i][4], s.handle), "hvdhip_batched_d2d_memcpy")
+        def pack(sets=sets, turn=turn):
+            i = turn[0] = (turn[0] + 1) % len(sets)
+            horovod_amd.check(copy(*sets[i][3], s.handle), "hvdhip_batched_d2d_memcpy")
 
-    sec = event_timed(gather_step, s, max(8, steps // 4), 4)
-    ab = 2 * slab + 2 * world * slab
-    return {"algorithmic_GB/s": round(ab / sec / 1e9, 1),
-            "algorithmic_frac_of_8TBps": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4),
-            "ms": round(sec * 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1), "entries": len(counts), "ranks": world,
-            "copies_per_step": len(counts) * (world + 1), "streams": 1, "replicas_rotated": len(sets)}
+        def unpack(sets=sets, turn=turn):
+            i = turn[0] = (turn[0] + 1) % len(sets)
+            horovod_amd.check(copy(*sets[i][4], s.handle), "hvdhip_batched_d2d_memcpy")
+
+        chunks = lambda sizes: sum((z + 4095) // 4096 for z in sizes)  # noqa: E731
+        cases += [
+            Case("ag.pack" + tag, "xfer_k<Copy<unsigned char>, 2, 1>", pack, 2 * slab,
+                 "this rank's %d entries (%d bytes) copied to its displacement in the allgather buffer; %d sets rotated"
+                 % (len(counts), slab, rotate), chunks([c * es for c in counts])),
+            Case("ag.unpack" + tag, "xfer_k<Copy<unsigned char>, 2, 0>", unpack, 2 * world * slab,
+                 "%d components (entry x rank) copied out of the %d-byte buffer into the entries' outputs; %d sets rotated"
+                 % (world * len(counts), world * slab, rotate), chunks(un_sz)),
+        ]
+    return cases
+
+
+def allgather_extra():
+    """The allgather fusion buffer's two copies as one step (pack + unpack), from their kernel loops."""
+    import torch
+    cases = build_cases("ag")
+    blocks = measure_cases(cases, steps=60, warmup=6)
+    release(cases)
+    del cases
+    torch.cuda.empty_cache()
+    out = {}
+    for tag, name in (("_small", "allgather_fusion_8ranks_128entries_6MB_slab"), ("", "allgather_fusion_8ranks_128entries_66MB_slab")):
+        pk = next(b for b in blocks if b["case"] == "ag.pack" + tag)
+        un = next(b for b in blocks if b["case"] == "ag.unpack" + tag)
+        ab = pk["algorithmic_bytes_per_launch"] + un["algorithmic_bytes_per_launch"]
+        sec = (pk["launch_us"] + un["launch_us"]) * 1e-6
+        out[name] = {"algorithmic_GB/s": round(ab / sec / 1e9, 1), "algorithmic_frac_of_8TBps": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4),
+                     "ms": round(sec * 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1), "streams": 1,
+                     "kernels": [pk, un], "traffic_profile": TRAFFIC_PROFILE["ag"],
+                     "note": "pack + unpack launch times added; each from its own back-to-back loop"}
+    return out
 
 
 def device_ceiling_extra(steps=20):
@@ -798,11 +1056,26 @@ def extras(headline_cases_block):
     out = {}
 
     def pipeline(name, shapes, tdt, bdt, std, peers, fraction, streams, replicas, steps, arrays=False, note=None,
-                 completion_events=None, record_with_unpack=False):
+                 completion_events=None, record_with_unpack=False, postscale=1.0):
         run = PipelineRun(shapes, tdt, bdt, std, peers, fraction, streams, replicas, arrays=arrays,
-                          completion_events=completion_events, record_with_unpack=record_with_unpack)
-        sec = timed(run.one_pass, run.sync, steps, max(2, steps // 10))
+                          completion_events=completion_events, record_with_unpack=record_with_unpack,
+                          postscale=postscale)
+        sec, each = timed_batches(run.one_pass, run.sync, steps, max(2, steps // 10))
         out[name] = pipeline_figures(run, sec, streams, note)
+        out[name]["ms_median_min_max"] = spread(each, 1e3, 4)
+        run.destroy()
+
+    def through_adapter(name, shapes, dt, std, slots, replicas, steps, beside):
+        run = AdapterRun(shapes, dt, std, slots, replicas)
+        sec, each = timed_batches(run.one_pass, run.sync, steps, max(2, steps // 10))
+        ab = run.algorithmic_bytes()
+        out[name] = {"algorithmic_GB/s": round(ab / sec / 1e9, 1),
+                     "algorithmic_frac_of_8TBps": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4), "ms": round(sec * 1e3, 4),
+                     "ms_median_min_max": spread(each, 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1),
+                     "cycles": len(run.groups), "streams": slots, "peers": 1, "replicas_rotated": len(run.reps),
+                     "vs_python_pipeline": round(out[beside]["ms"] / (sec * 1e3), 4),
+                     "note": "every response through the C++ adapter's GPUAllreduce::Execute on %d stream slot(s), completion "
+                             "on finalizer threads; vs_python_pipeline = time of %s / this time" % (slots, beside)}
         run.destroy()
 
     def kernels(name, cfg):
@@ -812,20 +1085,22 @@ def extras(headline_cases_block):
         del cases
         torch.cuda.empty_cache()
         out[name]["kernels"] = blocks
-        out[name]["roofline"] = max(blocks, key=lambda b: b["launch_us"])
+        out[name]["roofline_case"] = max((b for b in blocks if "+" not in b["case"]), key=lambda b: b["launch_us"])["case"]
         out[name]["traffic_profile"] = TRAFFIC_PROFILE.get(cfg.rstrip("h"))
 
     # C1 on two streams (the headline is the one-stream figure); its kernel blocks come from the headline
+    pipeline("c1_resnet50_fp32_one_stream", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0, 1, 4, 200,
+             completion_events=True, record_with_unpack=True,
+             note="the headline pipeline with the completion event of every cycle bound to its unpack kernel "
+                  "(hvdhip_fusion_unpack_record) and waited for by the host: what the adapter's Execute queues")
+    through_adapter("c1_resnet50_fp32_one_slot_through_the_adapter", W.resnet50_shapes(), F32, 1e-3, 1, 4, 200,
+                    "c1_resnet50_fp32_one_stream")
     pipeline("c1_resnet50_fp32_two_streams", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0, 2, 4, 200)
     out["c1_resnet50_fp32_two_streams"]["kernels"] = headline_cases_block
     pipeline("c1_resnet50_fp32_one_stream_completion_events", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0, 1, 4, 200,
              completion_events=True,
              note="the headline pipeline with a pooled completion event recorded behind every cycle and waited for by "
                   "the host, as GPUOpContext::FinalizeGPUQueue does once per response (ops/gpu_operations.cc:50-98)")
-    pipeline("c1_resnet50_fp32_one_stream_completion_events_with_unpack", W.resnet50_shapes(), F32, F32, 1e-3, 1, 1.0,
-             1, 4, 200, completion_events=True, record_with_unpack=True,
-             note="the same with the event bound to the unpack kernel's own completion (hvdhip_fusion_unpack_record) "
-                  "instead of recorded behind it")
 
     # C2: fusion stress, pack + unpack, 200 repetitions
     stress = [(c,) for c in W.stress_counts(seed=3)]
@@ -850,9 +1125,11 @@ def extras(headline_cases_block):
     except Exception as e:  # pragma: no cover
         out["c2_fusion_stress"]["execute_vs_per_tensor_copies"] = {"error": "%s: %s" % (type(e).__name__, e)}
 
-    # C3: BERT-large fp32 -> fp16, 7 peers on the 1/8 share
+    # C3: BERT-large fp32 -> fp16, 7 peers on the 1/8 share; postscale 1.0 and a non-trivial power of two
     pipeline("c3_bert_large_fp32_to_fp16_7peers_eighth_share", W.bert_large_shapes(), F32, F16, 1e-4, 7, 0.125, 1, 1, 20)
     kernels("c3_bert_large_fp32_to_fp16_7peers_eighth_share", "c3")
+    pipeline("c3_bert_large_postscale_4", W.bert_large_shapes(), F32, F16, 1e-4, 7, 0.125, 1, 1, 20, postscale=4.0,
+             note="the same pipeline with postscale 4.0 in the widening unpack (the kernel multiplies either way)")
     pipeline("c3_bert_large_two_streams", W.bert_large_shapes(), F32, F16, 1e-4, 7, 0.125, 2, 1, 20)
 
     # C4: Adasum combine, fp32 (the configuration) and fp16
@@ -864,25 +1141,77 @@ def extras(headline_cases_block):
         torch.cuda.empty_cache()
         b = blocks[0]
         out[name] = {"algorithmic_GB/s": b["achieved"], "algorithmic_frac_of_8TBps": b["frac"],
-                     "ms": round(b["launch_us"] / 1e3, 4), "algorithmic_MB": round(b["algorithmic_bytes_per_launch"] / 1e6, 1),
-                     "replicas_rotated": 4, "kernels": blocks, "roofline": b, "traffic_profile": TRAFFIC_PROFILE["c4"],
+                     "ms": round(b["launch_us"] / 1e3, 4), "ms_median_min_max": [round(x / 1e3, 4) for x in b["launch_us_median_min_max"]],
+                     "algorithmic_MB": round(b["algorithmic_bytes_per_launch"] / 1e6, 1),
+                     "replicas_rotated": 4, "kernels": blocks, "roofline_case": b["case"], "traffic_profile": TRAFFIC_PROFILE["c4"],
                      "note": "two launches timed together with HIP events; per-kernel durations and traffic are in the profile"}
 
-    # C5: GPT-2 XL fp16 on two streams (the configuration), on one, and through the array-taking entry points
+    # C5: GPT-2 XL fp16 on two streams (the configuration), on one, through the array-taking entry points
+    # and through the adapter on two stream slots
     pipeline("c5_gpt2_xl_fp16_two_streams", W.gpt2_xl_shapes(), F16, F16, 1e-3, 1, 1.0, 2, 1, 5)
     kernels("c5_gpt2_xl_fp16_two_streams", "c5")
+    through_adapter("c5_gpt2_xl_fp16_two_slots_through_the_adapter", W.gpt2_xl_shapes(), F16, 1e-3, 2, 1, 5,
+                    "c5_gpt2_xl_fp16_two_streams")
     pipeline("c5_gpt2_xl_fp16_one_stream", W.gpt2_xl_shapes(), F16, F16, 1e-3, 1, 1.0, 1, 1, 5)
     pipeline("c5_gpt2_xl_fp16_array_entry_points", W.gpt2_xl_shapes(), F16, F16, 1e-3, 1, 1.0, 2, 1, 5, arrays=True,
              note="pack and unpack of every cycle through hvdhip_batched_scaled_d2d_memcpy (the by-value launchers "
                   "of ops/gpu_operations.cc:186-206) instead of explicit plans: 96 distinct copy sets per step, "
                   "their tables resident in the library's cache after the first step")
 
-    out["allgather_fusion_8ranks_pack_unpack"] = allgather_extra(200)
+    out.update(allgather_extra())
     out["device_copy_1GiB_three_ways"] = device_ceiling_extra()
     return out
 
 
 # ----------------------------------------------------------------------------------------------
+# output: one compact JSON line on stdout (it has to fit a reader's 8 KB window), everything on stderr
+# ----------------------------------------------------------------------------------------------
+
+KERNEL_COLUMNS = ["case", "kernel", "launch_us", "us_median", "us_min", "us_max", "frac_of_8TBps",
+                  "algorithmic_B", "traffic_B", "in_pipeline_us"]
+PIPELINE_COLUMNS = ["algorithmic_GB/s", "frac_of_8TBps", "ms", "ms_median", "ms_min", "ms_max", "streams", "cpu_GB/s_1core"]
+
+
+def kernel_row(b):
+    m = b.get("launch_us_median_min_max") or [None, None, None]
+    return [b["case"], b["kernel"], b["launch_us"], m[0], m[1], m[2], b["frac"], b["algorithmic_bytes_per_launch"],
+            b.get("traffic"), b.get("in_pipeline_us")]
+
+
+def compact(result):
+    """The line for stdout: the contract's keys in full, every other configuration as one row per
+    pipeline and one row per kernel loop (columns named once)."""
+    out = {k: v for k, v in result.items() if k != "extra"}
+    out["config"] = {k: v for k, v in result["config"].items() if k != "value_is"}
+    extra = result.get("extra")
+    if not extra:
+        return out
+    if "error" in extra:
+        out["extra"] = extra
+        return out
+    pipes, rows, seen = {}, [], set()
+    for name, d in extra.items():
+        if not isinstance(d, dict):
+            continue
+        if "algorithmic_GB/s" in d:
+            m = d.get("ms_median_min_max") or [None, None, None]
+            pipes[name] = [d["algorithmic_GB/s"], d["algorithmic_frac_of_8TBps"], d["ms"], m[0], m[1], m[2],
+                           d.get("streams"), d.get("cpu_GB/s")]
+            if "vs_python_pipeline" in d:
+                pipes[name].append(d["vs_python_pipeline"])
+        for b in d.get("kernels", []):
+            if b["case"] not in seen:
+                seen.add(b["case"])
+                rows.append(kernel_row(b))
+    out["extra"] = {"pipeline_columns": PIPELINE_COLUMNS + ["(adapter rows: python pipeline's ms / this ms)"],
+                    "pipelines": pipes, "kernel_columns": KERNEL_COLUMNS, "kernels": rows}
+    ex = extra.get("c2_fusion_stress", {}).get("execute_vs_per_tensor_copies")
+    if ex:
+        out["extra"]["c2_execute_vs_per_tensor_copies"] = ex
+    if "cpu_error" in extra:
+        out["extra"]["cpu_error"] = extra["cpu_error"]
+    return out
+
 
 def main():
     args = parse()
@@ -903,13 +1232,22 @@ def main():
     stream = stream_pair()[0]
     F32 = DTYPE["float32"]
     if args.calibrate:
-        from horovod_amd import host as H
+        # Two plain 256 MiB device copies that are none of the library's kernels: the runtime's
+        # hipMemcpyAsync (its own copy kernel) and an elementwise kernel of torch.  Each reads exactly
+        # 262,144 KiB and writes exactly 262,144 KiB; what rocprofv3's FETCH_SIZE and WRITE_SIZE read
+        # for them gives the factors that turn those counters into bytes.
         n = 256 << 20
-        a = torch.zeros(n, dtype=torch.uint8, device="cuda")
+        a = randn_bytes(n, torch.float32, 1.0, 77)
         b = torch.empty(n, dtype=torch.uint8, device="cuda")
         torch.cuda.synchronize()
+        memcpy = horovod_amd.lib().hvdhip_memcpy_async
+        ext = torch.cuda.ExternalStream(stream.handle.value)
         for _ in range(args.warmup + args.steps):
-            H.batched_d2d_memcpy([b.data_ptr()], [a.data_ptr()], [n], stream)
+            horovod_amd.check(memcpy(b.data_ptr(), a.data_ptr(), n, 3, stream.handle), "hvdhip_memcpy_async")
+        stream.synchronize()
+        for _ in range(args.warmup + args.steps):
+            with torch.cuda.stream(ext):
+                torch.mul(a.view(torch.float32), 1.0, out=b.view(torch.float32))
         stream.synchronize()
         return
 
@@ -932,21 +1270,18 @@ def main():
         for _ in range(REPS):
             run.one_pass()
 
-    sec = timed(step, run.sync, args.steps, args.warmup)
+    sec, each = timed(step, run.sync, args.steps, args.warmup, stream=stream)
     ab = run.algorithmic_bytes()
     value = REPS * ab / sec / 1e9
     payload = 4 * sum(run.counts)
-    config = {"workload": "C1: ResNet-50 fp32 gradients, 161 tensors, 25,557,032 elements, N(0,1e-3); fused by the "
-                          "reference's planner at a 64 MiB threshold into %d cycles; per cycle pack with prescale 0.125 "
-                          "-> reduce-sum of the whole buffer with one peer buffer resident on the device -> unpack "
-                          "(postscale 1.0); all on one stream, the stream slot's one persistent fusion buffer; the "
-                          "tensor sets (inputs, outputs, peers) rotate over %d replicas so that no pass finds its "
-                          "inputs in the 256 MB Infinity Cache" % (len(run.pipe.cycles), len(run.reps)),
+    config = {"workload": "C1: ResNet-50 fp32 gradients, 161 tensors, 25,557,032 elements, N(0,1e-3); fused at a 64 MiB "
+                          "threshold into %d cycles; per cycle pack with prescale 0.125 -> reduce-sum of the whole buffer "
+                          "with one peer buffer on the device -> unpack (postscale 1.0); one stream, one persistent fusion "
+                          "buffer; tensor sets rotate over %d replicas" % (len(run.pipe.cycles), len(run.reps)),
               "tensors": len(run.counts), "payload_bytes": payload, "cycles": len(run.pipe.cycles),
               "cycle_buffer_bytes": [c.plan.buffer_len for c in run.pipe.cycles], "fusion_threshold": W.FUSION_THRESHOLD,
               "peers": 1, "prescale": 0.125, "postscale": 1.0, "passes_per_step": REPS,
-              "algorithmic_bytes_per_pass": ab, "algorithmic_bytes_per_step": REPS * ab, "replicas_rotated": len(run.reps),
-              "streams": 1,
+              "algorithmic_bytes_per_step": REPS * ab, "replicas_rotated": len(run.reps), "streams": 1,
               "value_is": "algorithmic bytes (pack P_in+P_buf, reduce 3C, unpack P_buf+P_out = 7P) / wall time; within a "
                           "cycle the fusion buffer passes from kernel to kernel through the Infinity Cache, so this is "
                           "not an HBM counter; the HBM claim is roofline.frac"}
@@ -959,15 +1294,21 @@ def main():
     del cases
     torch.cuda.empty_cache()
     roofline = dict(next(b for b in blocks if b["case"] == "c1.reduce"))
-    roofline["why_this_kernel"] = ("the reduce-sum takes the largest share of the pipeline's kernel time (3C of the "
-                                   "7P algorithmic bytes)")
+    roofline.pop("timed", None)
+    roofline["why_this_kernel"] = "the reduce-sum takes the largest share of the pipeline's kernel time (3C of 7P bytes)"
 
     result = {
         "metric": "achieved HBM GB/s (% of 8 TB/s) for fused pack+scale+reduce+unpack; Adasum GB/s",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(sec * 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic", "config": config,
+        # `value` counts algorithmic bytes over wall time; these three name what is what
+        "value_kind": "algorithmic GB/s of the whole pipeline (buffer hand-overs through the Infinity Cache included)",
+        "hbm_GB/s": round(roofline["traffic"] / (roofline["launch_us"] * 1e-6) / 1e9, 1) if roofline.get("traffic") else None,
+        "hbm_GB/s_is": "counter-derived HBM bytes per launch of the roofline kernel (profiles/) / its launch time in this run",
         "algorithmic_frac_of_8TBps": round(value / HBM_PEAK_GBS, 4),
+        "ms_per_step_median_min_max": spread(each, 1e3, 5),
+        "ms_per_step_from": "HIP event pair around each of the %d timed steps, on the pipeline's stream" % args.steps,
         "roofline": roofline,
         "traffic_profile": TRAFFIC_PROFILE["c1"],
     }
@@ -985,7 +1326,12 @@ def main():
                     result["extra"][name].update(v)
             except Exception as e:  # pragma: no cover
                 result["extra"]["cpu_error"] = "%s: %s" % (type(e).__name__, e)
-    print(json.dumps(result))
+    # everything, with the descriptions of what was timed, for whoever keeps stderr
+    print("DETAIL " + json.dumps(result), file=sys.stderr, flush=True)
+    line = json.dumps(compact(result), separators=(",", ":"))
+    if len(line) > 8000:
+        print("note: the stdout line is %d bytes" % len(line), file=sys.stderr)
+    print(line)
 
 
 if __name__ == "__main__":

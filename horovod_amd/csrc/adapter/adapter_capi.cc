@@ -47,6 +47,7 @@ struct Harness {
   std::deque<Op> ops;  // index = ticket; a deque so that queued entries stay where they are
   int completed = 0;
   std::vector<Prepared> prepared;
+  bool borrowed_streams = false;  // the streams belong to the caller: not to be destroyed with the context
 };
 
 int report(const std::exception& e, char* err, size_t errlen) {
@@ -160,12 +161,30 @@ void* hvd_adapter_create(int num_streams, int batch_d2d_memcopies, int enable_as
                                num_streams);
 }
 
+// Hands the context one existing stream per stream slot (device 0) instead of letting it create its
+// own at first use, as gpu_context.streams is filled by whoever gets there first in the reference
+// (ops/gpu_operations.cc:30-39).  Streams map onto a few hardware queues in the order they are
+// created; a process that wants two slots to overlap creates their streams early and hands them over.
+// The streams stay the caller's.
+int hvd_adapter_use_streams(void* handle, void* const* streams) {
+  Harness* h = static_cast<Harness*>(handle);
+  for (int slot = 0; slot < h->state.num_nccl_streams; ++slot) h->context.streams[(size_t)slot][0] = streams[slot];
+  h->borrowed_streams = true;
+  return 0;
+}
+
 void hvd_adapter_destroy(void* handle) {
   Harness* h = static_cast<Harness*>(handle);
   if (!h) return;
   h->context.finalizer_thread_pool.reset();  // the callbacks of queued responses run before the harness goes
   delete h->allreduce;
   delete h->adasum;
+  if (h->borrowed_streams) {
+    for (auto& per_device : h->context.streams) {
+      for (auto& kv : per_device) hvdhip_stream_synchronize(kv.second);
+      per_device.clear();
+    }
+  }
   delete h;  // the context's destructor gives its streams back
 }
 

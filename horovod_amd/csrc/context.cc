@@ -81,10 +81,21 @@ uint32_t chunk_bytes(Family f) {
     return 0u;
   }();
   if (forced) return forced;
+  // HVDHIP_UNPACK_CHUNK_BYTES: the unpack tables alone.
+  static uint32_t forced_unpack = [] {
+    const char* e = getenv("HVDHIP_UNPACK_CHUNK_BYTES");
+    if (e) {
+      long x = strtol(e, nullptr, 10);
+      if (x >= 4096 && x <= (1 << 24) && x % 4096 == 0) return (uint32_t)x;
+    }
+    return 0u;
+  }();
+  if (forced_unpack && f == Family::kUnpack) return forced_unpack;
 #endif
   switch (f) {
   case Family::kXfer: return kXferChunkBytes;
   case Family::kXferNarrowing: return kXferNarrowingChunkBytes;
+  case Family::kUnpack: return kUnpackChunkBytes;
   case Family::kReduce: return kReduceChunkBytes;
   default: return kAdasumChunkBytes;
   }
@@ -113,6 +124,7 @@ int upload_chunks(const std::vector<Chunk>& chunks, DevTables* out) {
   out->alloc = dev;
   out->chunks = static_cast<Chunk*>(dev);
   out->nchunks = (uint32_t)chunks.size();
+  out->nlaunch = out->nchunks;
   return 0;
 }
 
@@ -157,6 +169,8 @@ XcdOrder xcd_order(uint64_t nblocks, uint32_t tile_bytes) {
 void fill_chunks(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t tensor_es,
                  uint32_t buffer_es, Chunk* out, uint64_t nchunks) {
   const uint32_t run = xcd_run(nchunks, chunk_units * (tensor_es > buffer_es ? tensor_es : buffer_es));
+  const uint64_t slots = table_slots(nchunks);
+  for (uint64_t i = nchunks / kLineGroup * kLineGroup; i < slots; ++i) out[i] = Chunk{0, 0, 0, 0, 0};  // the padded last group
   uint64_t index = 0;
   for (const Seg& s : segs) {
     const uint64_t nbytes = s.n * buffer_es;
@@ -168,7 +182,7 @@ void fill_chunks(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t te
       c.off = s.off + start * buffer_es;
       c.n = (uint32_t)(left < chunk_units ? left : chunk_units);
       c.pad = left <= chunk_units ? (uint32_t)((16 - (nbytes & 15)) & 15) : 0;
-      out[xcd_slot(index++, nchunks, run)] = c;
+      out[line_slot((uint32_t)xcd_slot(index++, nchunks, run))] = c;
     }
   }
 }
@@ -178,9 +192,11 @@ int build_tables(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t te
   if (chunk_units == 0) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "chunk_units is zero");
   const uint64_t nchunks = count_chunks(segs, chunk_units);
   if (nchunks == ~0ull) return fail(HVDHIP_ERR_TOO_LARGE, "plan needs more than 2^23 workgroups");
-  std::vector<Chunk> chunks((size_t)nchunks);
+  std::vector<Chunk> chunks((size_t)table_slots(nchunks));
   fill_chunks(segs, chunk_units, tensor_es, buffer_es, chunks.data(), nchunks);
-  return upload_chunks(chunks, out);
+  int rc = upload_chunks(chunks, out);
+  if (rc == 0) out->nchunks = (uint32_t)nchunks;
+  return rc;
 }
 
 int free_tables(DevTables* t) {

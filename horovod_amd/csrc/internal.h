@@ -74,9 +74,10 @@ constexpr uint64_t kMaxWorkgroups = 1ull << 23;
 // The Adasum reduction pays a workgroup-wide tree per chunk and prefers 16 KiB.
 // (A build with -DHVDHIP_TUNING reads HVDHIP_CHUNK_BYTES to override all of them; the shipped
 // library reads nothing.)
-enum class Family { kXfer, kXferNarrowing, kReduce, kAdasum };
+enum class Family { kXfer, kXferNarrowing, kUnpack, kReduce, kAdasum };
 constexpr uint32_t kXferChunkBytes = 4096;
 constexpr uint32_t kXferNarrowingChunkBytes = 8192;  // fp32 -> fp16 pack: 32 bytes in, 16 out per lane
+constexpr uint32_t kUnpackChunkBytes = 4096;  // every unpack, same-width or widening (a plan keeps a second table when this differs from its pack's)
 constexpr uint32_t kReduceChunkBytes = 4096;
 constexpr uint32_t kAdasumChunkBytes = 16384;
 uint32_t chunk_bytes(Family f);
@@ -193,6 +194,19 @@ struct Seg {
   uint64_t n;
 };
 
+// Where workgroup b finds its entry in a transfer table.  Four 32-byte entries share a 128-byte
+// cache line, and workgroups b, b + 1, b + 2, b + 3 run on four different XCDs, each with an L2 of
+// its own: read in workgroup order, every line is fetched from memory four times (128 bytes per
+// workgroup for a 32-byte entry, +1.6 % read traffic on a 4 KiB chunk).  So within each group of
+// 32 workgroups the four that share an XCD (b, b + 8, b + 16, b + 24: consecutive on that XCD)
+// read the four entries of one line.  Tables are padded to a multiple of 32 entries with empty
+// chunks (n = 0), and that many workgroups are launched, so the mapping needs no bounds check and
+// no argument: nothing stands between a workgroup's start and the load of its entry but three
+// scalar instructions.
+constexpr uint32_t kLineGroup = 32;
+inline uint64_t table_slots(uint64_t nchunks) { return (nchunks + kLineGroup - 1) / kLineGroup * kLineGroup; }
+__host__ __device__ inline uint32_t line_slot(uint32_t b) { return (b & ~31u) | ((b & 7u) << 2) | ((b >> 3) & 3u); }
+
 // One workgroup's share, self-contained so that a workgroup needs a single
 // 32-byte scalar load before it can issue its data loads.  All three
 // locations already point at the chunk's first element.
@@ -209,7 +223,8 @@ static_assert(sizeof(Chunk) == 32, "Chunk is loaded as eight dwords");
 struct DevTables {
   void* alloc = nullptr;
   Chunk* chunks = nullptr;
-  uint32_t nchunks = 0;
+  uint32_t nchunks = 0;  // chunks with work in them
+  uint32_t nlaunch = 0;  // entries in the table = workgroups to launch (transfer tables: padded to 32)
 };
 
 // Cuts every segment into chunks of at most chunk_units elements and uploads
@@ -220,7 +235,8 @@ int build_tables(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t te
                  uint32_t buffer_es, DevTables* out);
 // The two halves of build_tables for callers that stage the table themselves:
 // the number of chunks the segments need (0xffffffffffffffff if over the
-// limit), and the fill of a caller-provided array of that many entries (in XCD order).
+// limit), and the fill of a caller-provided array of table_slots(nchunks) entries: XCD order,
+// each at the line_slot of its workgroup, the rest empty.
 uint64_t count_chunks(const std::vector<Seg>& segs, uint32_t chunk_units);
 void fill_chunks(const std::vector<Seg>& segs, uint32_t chunk_units, uint32_t tensor_es,
                  uint32_t buffer_es, Chunk* out, uint64_t nchunks);
@@ -248,7 +264,7 @@ void copy_cache_forget_stream(hipStream_t stream);
 // Destroys the single-layer Adasum plans kept for `stream` (idle, about to be destroyed).
 void adasum_forget_stream(hipStream_t stream);
 
-// Uploads a ready-made chunk table.
+// Uploads a ready-made chunk table; every entry is launched (nlaunch = nchunks = its size).
 int upload_chunks(const std::vector<Chunk>& chunks, DevTables* out);
 int free_tables(DevTables* t);
 

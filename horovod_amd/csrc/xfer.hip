@@ -183,7 +183,8 @@ __device__ __forceinline__ void stream_range(gptr<const typename Op::S> src,
 
 enum Mode { kPack = 0, kUnpack = 1, kDirect = 2 };
 
-// One workgroup per chunk-table entry.
+// One workgroup per chunk-table entry (entry line_slot(b) for workgroup b; the entries that pad
+// the table to a multiple of 32 are empty and their workgroups leave at once).
 //   kPack:   src = chunk.tensor,      dst = base + chunk.off (pad bytes zeroed)
 //   kUnpack: src = base + chunk.off,  dst = chunk.output
 //   kDirect: src = chunk.tensor,      dst = chunk.output
@@ -192,7 +193,7 @@ __global__ __launch_bounds__(kWG) void xfer_k(const Chunk* __restrict__ chunks, 
                                               typename Op::P p) {
   typedef typename Op::S S;
   typedef typename Op::D D;
-  const Chunk c = chunks[blockIdx.x];
+  const Chunk c = chunks[line_slot(blockIdx.x)];
   const uint64_t src_addr = (MODE == kUnpack) ? base + c.off : c.tensor;
   const uint64_t dst_addr = (MODE == kPack) ? base + c.off : c.output;
   stream_range<Op, ST>(as_global<const S>(src_addr), as_global<D>(dst_addr), c.n, p);
@@ -233,7 +234,7 @@ int launch_xfer(const DevTables& t, uint64_t base, typename Op::P p, hipStream_t
                         : MODE == kPack ? (converting ? Stores::kPackNarrowing : Stores::kPack)
                                         : (converting ? Stores::kUnpackWidening : Stores::kUnpack);
   const hipError_t status = with_store_policy(family, [&](auto st) {
-    return launch_with(completion, xfer_k<Op, MODE, decltype(st)::value>, t.nchunks, stream, t.chunks, base, p);
+    return launch_with(completion, xfer_k<Op, MODE, decltype(st)::value>, t.nlaunch, stream, t.chunks, base, p);
   });
   HVDHIP_CHECK_LAUNCH("xfer_k", status);
   return 0;
@@ -554,7 +555,7 @@ int cached_tables(CopyCache& c, void* const* out, const void* const* in, const s
   const uint32_t chunk_units = chunk_bytes(Family::kXfer) / unit;
   const uint64_t nchunks = count_chunks(segs, chunk_units);
   if (nchunks == ~0ull) return fail(HVDHIP_ERR_TOO_LARGE, "the copies need more than 2^23 workgroups");
-  const size_t bytes = (size_t)nchunks * sizeof(Chunk);
+  const size_t bytes = (size_t)table_slots(nchunks) * sizeof(Chunk);
   while (!c.lru.empty() && (c.lru.size() >= c.max_entries || c.bytes + bytes > c.max_bytes)) {
     int rc = evict_one(c);
     if (rc) return rc;
@@ -589,6 +590,7 @@ int cached_tables(CopyCache& c, void* const* out, const void* const* in, const s
   entry.tables.alloc = nullptr;
   entry.tables.chunks = static_cast<Chunk*>(entry.buf.dev);
   entry.tables.nchunks = (uint32_t)nchunks;
+  entry.tables.nlaunch = (uint32_t)table_slots(nchunks);
   entry.build_stream = stream;
   entry.gathers = n > 1;
   for (int i = 0; i + 1 < n && entry.gathers; ++i) {
@@ -652,8 +654,9 @@ struct hvdhip_fusion_plan {
   int buffer_dtype = 0;
   int64_t buffer_len = 0;
   std::vector<int64_t> offsets;
-  DevTables tables;       // pack (and unpack, when not converting)
-  DevTables unpack_tables;  // converting plans only: unpack prefers smaller chunks than pack
+  DevTables tables;         // pack, and unpack when both are cut into chunks of the same size
+  DevTables unpack_tables;  // unpack, when it prefers another chunk size than pack (the converting plans)
+  bool own_unpack_tables = false;
   bool converting = false;
 };
 
@@ -801,9 +804,11 @@ int hvdhip_fusion_plan_create(const void* const* tensors, void* const* outputs,
   // every same-width transfer with 4 KiB.
   const uint32_t wide = (uint32_t)std::max(ts, bs);
   const uint32_t pack_bytes = p->converting ? chunk_bytes(Family::kXferNarrowing) : chunk_bytes(Family::kXfer);
+  const uint32_t unpack_bytes = chunk_bytes(Family::kUnpack);
   int rc = build_tables(segs, pack_bytes / wide, (uint32_t)ts, (uint32_t)bs, &p->tables);
-  if (rc == 0 && p->converting) {
-    rc = build_tables(segs, chunk_bytes(Family::kXfer) / wide, (uint32_t)ts, (uint32_t)bs, &p->unpack_tables);
+  p->own_unpack_tables = unpack_bytes != pack_bytes;
+  if (rc == 0 && p->own_unpack_tables) {
+    rc = build_tables(segs, unpack_bytes / wide, (uint32_t)ts, (uint32_t)bs, &p->unpack_tables);
     if (rc) free_tables(&p->tables);
   }
   if (rc) {
@@ -873,12 +878,13 @@ int unpack(hvdhip_fusion_plan* plan, const void* fusion_buffer, double scale_fac
   const uint64_t base = (uint64_t)(uintptr_t)fusion_buffer;
   int rc;
   if (plan->buffer_dtype != plan->tensor_dtype) {
-    rc = launch_xfer<UnpackF16F32, kUnpack>(plan->unpack_tables, base, {fp16_scale_factor(scale_factor)}, s, false,
-                                            completion);
+    rc = launch_xfer<UnpackF16F32, kUnpack>(plan->own_unpack_tables ? plan->unpack_tables : plan->tables, base,
+                                            {fp16_scale_factor(scale_factor)}, s, false, completion);
   } else {
     if (scale_factor != 1.0 && !scalable(plan->tensor_dtype))
       return fail(HVDHIP_ERR_UNSUPPORTED_DTYPE, "dtype %d cannot be scaled", plan->tensor_dtype);
-    rc = launch_same_dtype<kUnpack>(plan->tables, base, scale_factor, plan->tensor_dtype, s, false, completion);
+    rc = launch_same_dtype<kUnpack>(plan->own_unpack_tables ? plan->unpack_tables : plan->tables, base, scale_factor,
+                                    plan->tensor_dtype, s, false, completion);
   }
   return rc ? rc : ok();
 }

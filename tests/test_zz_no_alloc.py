@@ -99,3 +99,71 @@ def test_largest_size_runs(gpu):
     gpu.sync()
     assert d_res.cpu().tolist() == [float(n)] * 3 + [0.5, 0.5]
     assert int((x != 1).sum()) == 0
+
+
+@pytest.mark.parametrize("chunks", [37, 700])
+def test_a_captured_call_replays_like_the_eager_one(gpu, chunks):
+    """The property the entry point exists for.  Under stream capture (torch's default, global mode)
+    an allocation, a free, a blocking copy or a synchronisation on any thread is refused, so a
+    call that did any of those would fail the capture; the recorded graph holds kernels only.  It is
+    replayed three times on fresh inputs, with eager work and synchronisations in between, and every
+    replay must equal the planned combine of the same inputs to the bit (vector, sums, coefficients).
+    37 chunks take the path that sums inside the scaled add, 700 the one with a sum launch of its own."""
+    import horovod_amd
+    n = chunks * 4096 - 5
+    side = torch.cuda.Stream()
+    s = horovod_amd.Stream(side.cuda_stream)
+    a = torch.zeros(n, device="cuda")
+    b = torch.zeros(n, device="cuda")
+    a2 = torch.zeros(n, device="cuda")
+    res = torch.zeros(5, dtype=torch.float64, device="cuda")
+    static = horovod_amd.lib().hvdhip_adasum_combine_static
+
+    def call():
+        horovod_amd.check(static(a.data_ptr(), b.data_ptr(), F32, n, res.data_ptr(), s.handle),
+                          "hvdhip_adasum_combine_static")
+
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        call()  # warm-up outside the capture: the scratch array's address is looked up on the first call
+        side.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            call()
+        side.synchronize()
+    gen = torch.Generator(device="cuda")
+    for replay in range(3):
+        gen.manual_seed(50 + replay)
+        a.copy_(torch.randn(n, generator=gen, device="cuda"))
+        b.copy_(0.3 * a + torch.randn(n, generator=gen, device="cuda"))
+        a2.copy_(a)
+        res.fill_(-1.0)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        want5 = _planned(gpu, a2, b, F32, n)  # eager, with its own plan and its own synchronisations
+        torch.cuda.synchronize()
+        assert torch.equal(a.view(torch.int32), a2.view(torch.int32)), "replay %d" % replay
+        assert np.array_equal(res.cpu().numpy().view(np.uint64), want5.view(np.uint64)), "replay %d" % replay
+        assert not torch.equal(a, b)
+
+
+def test_eager_calls_leave_the_device_memory_as_it_was(gpu):
+    """hipMemGetInfo's free bytes before and after 100 calls (after one warm-up call): the entry
+    point takes nothing from the device allocator, whatever the sizes it is called with."""
+    rng = np.random.default_rng(43)
+    sizes = [1, 4096 * 37 - 5, 4096 * 700 + 1234, 1 << 22, 17]
+    n_max = max(sizes)
+    a, b = _pair(rng, n_max, np.float32)
+    d_a, d_b = gpu.upload(a), gpu.upload(b)
+    d_res = torch.zeros(5, dtype=torch.float64, device="cuda")
+    _static(gpu, d_a, d_b, F32, sizes[1], d_res)
+    gpu.sync()
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for i in range(100):
+        _static(gpu, d_a, d_b, F32, sizes[i % len(sizes)], d_res)
+    gpu.sync()
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before
