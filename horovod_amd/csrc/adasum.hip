@@ -779,12 +779,19 @@ namespace {
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mu;
 unsigned char* g_scratch_ptr[kMaxDevices];  // the device address of `scratch`, per device
+// All calls on a device share its one array, so each call is ordered behind the one before it:
+// an event is recorded behind a call's last kernel, and a call on another stream makes its stream
+// wait for that event first.  The event is made once per device, with the address look-up.
+hipEvent_t g_scratch_last_use[kMaxDevices];
+hipStream_t g_scratch_last_stream[kMaxDevices];
+bool g_scratch_used[kMaxDevices];
 
 // The address of the current device's copy of `scratch`.  In host code the array's name is only
 // a handle for the symbol; every use below goes through this pointer.
-int static_scratch(unsigned char** out) {
+int static_scratch(unsigned char** out, int* device_out) {
   int device = 0;
   HVDHIP_CHECK(hipGetDevice(&device));
+  *device_out = device;
   if (device < 0 || device >= kMaxDevices)
     return fail(HVDHIP_ERR_INVALID_ARGUMENT, "device %d is beyond the %d devices this entry point serves", device,
                 kMaxDevices);
@@ -793,6 +800,7 @@ int static_scratch(unsigned char** out) {
     void* p = nullptr;
     HVDHIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
     if (!p) return fail(HVDHIP_ERR_INVALID_ARGUMENT, "hipGetSymbolAddress returned no address for the scratch array");
+    HVDHIP_CHECK(hipEventCreateWithFlags(&g_scratch_last_use[device], hipEventDisableTiming | hipEventDisableSystemFence));
     g_scratch_ptr[device] = static_cast<unsigned char*>(p);
   }
   *out = g_scratch_ptr[device];
@@ -813,7 +821,8 @@ int hvdhip_adasum_combine_static(void* a, const void* b, int dtype, int count, d
                 "count %d needs %llu chunks of %u elements; hvdhip_adasum_combine_static holds %u (use a plan)",
                 count, (unsigned long long)nchunks, chunk_units, kStaticMaxChunks);
   unsigned char* base = nullptr;
-  int rc = static_scratch(&base);
+  int device = 0;
+  int rc = static_scratch(&base, &device);
   if (rc) return rc;
   // A plan-shaped view of the scratch: nothing here is owned, nothing is freed.
   hvdhip_adasum_plan view;
@@ -830,6 +839,16 @@ int hvdhip_adasum_combine_static(void* a, const void* b, int dtype, int count, d
   rc = check_vectors(&view, a, b);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  // One call at a time per device, on the host (the launches of two calls must not interleave) and
+  // on the device (behind the last call's kernels).  A stream that is being captured takes neither
+  // the wait nor the record: events recorded outside a capture cannot be waited for inside one, so
+  // whoever launches the graph orders it against other calls.
+  std::lock_guard<std::mutex> one_call(g_scratch_mu);
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  HVDHIP_CHECK(hipStreamIsCapturing(s, &capture));
+  const bool eager = capture == hipStreamCaptureStatusNone;
+  if (eager && g_scratch_used[device] && g_scratch_last_stream[device] != s)
+    HVDHIP_CHECK(hipStreamWaitEvent(s, g_scratch_last_use[device], 0));
   // The array keeps what the last call left: the tables are rewritten for this count, and every
   // partial sum that is read is written first by this call's first pass.
   const uint32_t run = xcd_run(nchunks, chunk_bytes(Family::kAdasum), true);
@@ -841,7 +860,13 @@ int hvdhip_adasum_combine_static(void* a, const void* b, int dtype, int count, d
   if (rc) return rc;
   rc = fused ? scaled_add_by_dtype<true>(&view, a, b, nullptr, 0., 0., s)
              : plan_scaled_add(&view, a, b, view.coeffs, 0., 0., s);
-  return rc ? rc : ok();
+  if (rc) return rc;
+  if (eager) {
+    HVDHIP_CHECK(hipEventRecord(g_scratch_last_use[device], s));
+    g_scratch_last_stream[device] = s;
+    g_scratch_used[device] = true;
+  }
+  return ok();
 }
 
 }  // extern "C"

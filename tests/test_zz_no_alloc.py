@@ -167,3 +167,40 @@ def test_eager_calls_leave_the_device_memory_as_it_was(gpu):
     torch.cuda.synchronize()
     free_after, _ = torch.cuda.mem_get_info()
     assert free_after == free_before
+
+
+def test_calls_from_two_streams_are_ordered_by_the_library(gpu):
+    """All calls on a device share one scratch array, so the library puts each behind the one
+    before it (an event behind every call, a stream wait in the next call from another stream).
+    Two streams call alternately, 40 times each, on vectors of their own and of different sizes
+    (one with a sum launch of its own, one that sums inside the scaled add), nothing synchronised in
+    between; each vector must come out exactly as 40 planned combines in a row leave it."""
+    import horovod_amd
+    rng = np.random.default_rng(44)
+    s1, s2 = horovod_amd.Stream(), horovod_amd.Stream()
+    sizes = (700 * 4096 + 99, 37 * 4096 - 5)
+    data = []
+    for n in sizes:
+        a, b = _pair(rng, n, np.float32)
+        data.append((gpu.upload(a), gpu.upload(a), gpu.upload(b), n))
+    static = horovod_amd.lib().hvdhip_adasum_combine_static
+    try:
+        torch.cuda.synchronize()
+        for _ in range(40):
+            for (d_a, _, d_b, n), s in zip(data, (s1, s2)):
+                horovod_amd.check(static(d_a.data_ptr(), d_b.data_ptr(), F32, n, None, s.handle),
+                                  "hvdhip_adasum_combine_static")
+        s1.synchronize()
+        s2.synchronize()
+        for d_a, d_ref, d_b, n in data:
+            plan = gpu.H.AdasumPlan([n], F32)
+            try:
+                for _ in range(40):
+                    plan.combine(d_ref.data_ptr(), d_b.data_ptr(), gpu.stream)
+                gpu.sync()
+            finally:
+                plan.destroy()
+            assert np.array_equal(gpu.download(d_a, np.uint32), gpu.download(d_ref, np.uint32)), n
+    finally:
+        s1.destroy()
+        s2.destroy()
