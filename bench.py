@@ -287,14 +287,11 @@ class Case:
     parts: for a call that launches several kernels, [(kernel, algorithmic bytes, algorithmic bytes read)] per
     kernel; reads: the algorithmic bytes read of a single-kernel call when that is not half of alg."""
 
-    def __init__(self, key, kernel, fn, alg, what, workgroups=None, cleanup=None, parts=None, follows=None, reads=None):
+    def __init__(self, key, kernel, fn, alg, what, workgroups=None, cleanup=None, parts=None, reads=None):
         self.key, self.kernel, self.fn, self.alg, self.what, self.workgroups = key, kernel, fn, alg, what, workgroups
         self.cleanup = cleanup  # destroys the plans behind fn (the closures hold the device memory)
         # per kernel of the call: (name, algorithmic bytes, of which read); a copy reads half of what it moves
         self.parts = parts or [(kernel, alg, alg // 2 if reads is None else reads)]
-        # (case of the first kernel alone, case of the second kernel alone) when fn launches the two back to
-        # back on the same buffer, so that the second finds its input in the Infinity Cache (informative)
-        self.follows = follows
 
 
 def cycle_cases(cfg, counts, tdtype, bdtype, std, peers, share_world, stream, pack_kernel, reduce_kernel,
@@ -397,8 +394,7 @@ def cycle_cases(cfg, counts, tdtype, bdtype, std, peers, share_world, stream, pa
                           "the reduce-sum and, right behind it on the same buffer, the unpack: the unpack's input comes "
                           "out of the Infinity Cache as in a cycle (a kernel trace gives each kernel's own duration)",
                           None, None, [(reduce_kernel, (peers + 2) * share * bs, (peers + 1) * share * bs),
-                                       (unpack_kernel, payload * (bs + ts), payload * bs)],
-                          follows=(cfg + ".reduce", cfg + ".unpack")))
+                                       (unpack_kernel, payload * (bs + ts), payload * bs)]))
     if peers >= 3:
         # The worst placement of a staging ring: the resident chunk and its peers exactly 8 MiB apart
         # (a 1/8 share of a 64 MiB buffer is 8 MiB), against the back-to-back placement above.
