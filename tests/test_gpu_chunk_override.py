@@ -36,6 +36,19 @@ def test_parity_with_64_kib_chunks(gpu):
     assert " passed" in tail and "failed" not in tail
 
 
+def test_parity_with_unpack_tables_of_their_own(gpu):
+    """HVDHIP_UNPACK_CHUNK_BYTES=8192: every plan then keeps a second chunk table for its unpack (as
+    the converting plans always do), cut into chunks of another size than its pack's."""
+    env = dict(os.environ, HVDHIP_UNPACK_CHUNK_BYTES="8192", HVDHIP_LIBRARY=TUNING)
+    cmd = [sys.executable, "-m", "pytest", "-q", "-x", "-m", "gpu", "--timeout", "300", "--timeout-method", "thread",
+           os.path.join(ROOT, "tests", "test_gpu_pack.py"), os.path.join(ROOT, "tests", "test_gpu_configs.py"),
+           "-p", "no:cacheprovider"]
+    r = subprocess.run(cmd, cwd=ROOT, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=900)
+    tail = r.stdout.decode(errors="replace")[-3000:]
+    assert r.returncode == 0, tail
+    assert " passed" in tail and "failed" not in tail
+
+
 @pytest.mark.parametrize("mask", ["0", "0x1ff"])
 def test_parity_with_every_kernel_family_on_one_store_policy(gpu, mask):
     env = dict(os.environ, HVDHIP_WRITE_THROUGH=mask, HVDHIP_LIBRARY=TUNING)
