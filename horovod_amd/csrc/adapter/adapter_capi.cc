@@ -48,6 +48,7 @@ struct Harness {
   int completed = 0;
   std::vector<Prepared> prepared;
   bool borrowed_streams = false;  // the streams belong to the caller: not to be destroyed with the context
+  std::vector<void*> next_ready_events;  // for the entries of the next response queued
 };
 
 int report(const std::exception& e, char* err, size_t errlen) {
@@ -78,6 +79,7 @@ int queue_response(Harness* h, std::vector<TensorTableEntry>& entries, double pr
     h->ops.back().queued_at = now_s();
   }
   for (auto& e : entries) {
+    e.ready_events = h->next_ready_events;
     e.callback = [h, ticket](const Status& status) {
       // what a framework's callback does with asynchronous completion: its own stream (here the
       // null stream) waits for the event (horovod/torch/mpi_ops_v2.cc:110-116)
@@ -95,6 +97,7 @@ int queue_response(Harness* h, std::vector<TensorTableEntry>& entries, double pr
       }
     };
   }
+  h->next_ready_events.clear();
   std::vector<const void*> p(peers, peers + npeers);
   try {
     h->allreduce->Execute(entries, prescale, postscale, p);
@@ -245,6 +248,15 @@ int hvd_adapter_execute_prepared(void* handle, int id, double prescale, double p
   } catch (const std::exception& e) {
     return report(e, err, errlen);
   }
+}
+
+// The framework's ready events (hipEvent_t) for every entry of the next response queued: what the
+// entries' ReadyEventList would hold.  All entries get the same events, as tensors produced by one
+// backward pass do.
+int hvd_adapter_next_ready_events(void* handle, void* const* events, int n) {
+  Harness* h = static_cast<Harness*>(handle);
+  h->next_ready_events.assign(events, events + n);
+  return 0;
 }
 
 int hvd_adapter_wait(void* handle, int ticket, char* err, size_t errlen) {

@@ -2,8 +2,10 @@
 #include "hvd_hip_adapter.h"
 
 #include <algorithm>
+#include <chrono>
 #include <stdexcept>
 #include <thread>
+#include <unordered_set>
 
 namespace horovod {
 namespace common {
@@ -418,11 +420,41 @@ void GPUAllreduce::ScaleBuffer(double scale_factor, const std::vector<TensorTabl
                                 Stream(entries));
 }
 
+void GPUAllreduce::WaitForData(std::vector<TensorTableEntry>& entries) {
+  if (global_state_->timeline_initialized) {
+    // the normal CPU syncing path: poll until every entry's events have completed
+    bool waited = false;
+    for (auto& e : entries) {
+      for (void* ev : e.ready_events) {
+        waited = true;
+        for (;;) {
+          int done = 0;
+          gpu_context_->ErrorCheck("hipEventQuery", hvdhip_event_query(ev, &done));
+          if (done) break;
+          std::this_thread::sleep_for(std::chrono::nanoseconds(100));
+        }
+      }
+    }
+    if (waited) {
+      std::lock_guard<std::mutex> guard(global_state_->timeline_mutex);
+      global_state_->timeline_activities.push_back(WAIT_FOR_DATA);
+    }
+    return;
+  }
+  // entries that were produced together share an event: wait for each one once
+  std::unordered_set<void*> event_set;
+  for (auto& e : entries)
+    for (void* ev : e.ready_events) event_set.insert(ev);
+  for (void* ev : event_set)
+    gpu_context_->ErrorCheck("hipStreamWaitEvent", hvdhip_stream_wait_event(*gpu_op_context_.stream, ev));
+}
+
 Status GPUAllreduce::Execute(std::vector<TensorTableEntry>& entries, double prescale_factor,
                              double postscale_factor, const std::vector<const void*>& peers) {
   auto& first_entry = entries[0];
   gpu_op_context_.InitGPU(entries);
   gpu_op_context_.InitGPUQueue(entries);
+  WaitForData(entries);
   const void* fused_input_data;
   void* buffer_data;
   size_t buffer_len;

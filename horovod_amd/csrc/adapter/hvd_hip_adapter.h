@@ -54,6 +54,7 @@ const std::string& DataType_Name(DataType value);     // common/message.cc:40-64
 typedef void* gpuStream_t;
 
 // Activity names of the stages on this path, common/common.h:73-105.
+#define WAIT_FOR_DATA "WAIT_FOR_DATA"
 #define QUEUE "QUEUE"
 #define MEMCPY_IN_FUSION_BUFFER "MEMCPY_IN_FUSION_BUFFER"
 #define MEMCPY_OUT_FUSION_BUFFER "MEMCPY_OUT_FUSION_BUFFER"
@@ -103,6 +104,9 @@ struct TensorTableEntry {
   // left at its default the entry travels as it is.
   int buffer_dtype = -1;
   DataType wire_dtype() const { return buffer_dtype < 0 ? dtype : (DataType)buffer_dtype; }
+  // ReadyEventList (common/common.h:262-300): events the framework recorded behind whatever produces
+  // the tensor; empty when the data is ready at enqueue time.
+  std::vector<void*> ready_events;
   // Called from a finalizer thread once the response has completed (or, with asynchronous
   // completion, once its last work has been queued); may be empty (common/common.cc:202-208).
   StatusCallback callback;
@@ -227,6 +231,11 @@ public:
   // response is queued; every entry's callback is called once it has completed.
   Status Execute(std::vector<TensorTableEntry>& entries, double prescale_factor, double postscale_factor,
                  const std::vector<const void*>& peers);
+
+  // NCCLAllreduce::WaitForData (ops/nccl_operations.cc:140-154): the op's stream waits for the
+  // entries' ready events, each once, with no host synchronisation; with the timeline on, the host
+  // polls them instead (HorovodOp::WaitForData, ops/collective_operations.cc:35-62).
+  void WaitForData(std::vector<TensorTableEntry>& entries);
 
   void MemcpyInFusionBuffer(const std::vector<TensorTableEntry>& entries, const void*& fused_input_data,
                             void*& buffer_data, size_t& buffer_len);

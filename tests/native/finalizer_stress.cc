@@ -286,6 +286,45 @@ void pool_semantics() {
   idle.wait_idle();  // no threads: nothing to wait for
 }
 
+// 8. WaitForData: the tensors are produced on another stream (a copy that takes 20 ms) with an event
+//    recorded behind it; Execute is called at once with that event as every entry's ready event and
+//    must not read the tensors before the producer has written them -- by a stream wait, or, with the
+//    timeline on, by polling on the host.
+void waits_for_the_producer() {
+  for (int timeline = 0; timeline < 2; ++timeline) {
+    Rig rig(1, 1, false, false, timeline != 0);
+    const std::vector<int> counts = {300, 5};
+    Response r;
+    build(r, 30 + timeline, counts);
+    // what the producer will write; the tensors hold something else until then
+    std::vector<std::vector<float>> produced = r.tensors;
+    for (auto& t : r.tensors)
+      for (auto& x : t) x = -12345.f;
+    void* producer = nullptr;
+    REQUIRE(hvdhip_set_device(0) == 0);
+    REQUIRE(hvdhip_stream_create(&producer) == 0);
+    void* ready = nullptr;
+    REQUIRE(hvdhip_event_acquire(producer, &ready) == 0);
+    fake_set_kernel_delay_us(20000);
+    for (size_t i = 0; i < counts.size(); ++i)
+      REQUIRE(hvdhip_memcpy_async(r.tensors[i].data(), produced[i].data(), produced[i].size() * 4, HVDHIP_MEMCPY_D2D, producer) == 0);
+    fake_set_kernel_delay_us(0);
+    REQUIRE(hvdhip_event_record(ready, producer) == 0);
+    for (auto& e : r.entries) e.ready_events = {ready};
+    rig.op->Execute(r.entries, 0.5, 1.0, {});
+    rig.context.finalizer_thread_pool.wait_idle();
+    REQUIRE(r.callbacks == 2 && r.failures == 0);
+    r.tensors = produced;  // check() reads the inputs from here
+    check(r, counts, 0.5f, 1.f, false);
+    if (timeline) {
+      std::lock_guard<std::mutex> g(rig.state.timeline_mutex);
+      REQUIRE(rig.state.timeline_activities.front() == WAIT_FOR_DATA);
+    }
+    REQUIRE(hvdhip_event_release(producer, ready) == 0);
+    REQUIRE(hvdhip_stream_destroy(producer) == 0);
+  }
+}
+
 }  // namespace
 
 int main() {
@@ -297,6 +336,7 @@ int main() {
   inline_completion();
   async_completion();
   elastic_and_timeline();
+  waits_for_the_producer();
   std::printf("finalizer ok\n");
   return 0;
 }

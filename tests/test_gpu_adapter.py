@@ -473,3 +473,46 @@ def test_a_run_of_responses_with_and_without_finalizer_threads(gpu, orc, adapter
         assert np.array_equal(got, orc.scale_buffer(v, 0.25, F32))
     finally:
         h.close()
+
+
+@pytest.mark.parametrize("timeline", [False, True])
+def test_execute_waits_for_the_entries_ready_events(gpu, orc, adapter, timeline):
+    """NCCLAllreduce::WaitForData (ops/nccl_operations.cc:140-154): the tensors are written on another
+    stream behind a kernel that spins for tens of milliseconds, with the framework's ready event
+    recorded behind the writes; Execute is called at once and must sum what the producer wrote, not
+    what the tensors held before -- through a stream wait, or with the timeline on through the
+    host's polling (ops/collective_operations.cc:35-62)."""
+    import torch
+    adapter.hvd_adapter_next_ready_events.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int]
+    adapter.hvd_adapter_set_timeline.argtypes = [ctypes.c_void_p, ctypes.c_int]
+    adapter.hvd_adapter_timeline.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]
+    counts = [70001, 5, 4096]
+    g = torch.Generator(device="cuda")
+    g.manual_seed(21)
+    fresh = [torch.randn(c, generator=g, device="cuda", dtype=torch.float32) for c in counts]
+    tensors = [torch.full((c,), -7.0, device="cuda", dtype=torch.float32) for c in counts]
+    outs = [torch.zeros(c, device="cuda", dtype=torch.float32) for c in counts]
+    side = torch.cuda.Stream()
+    ready = torch.cuda.Event()
+    torch.cuda.synchronize()
+    h = Harness(adapter, gpu, num_streams=1)
+    try:
+        adapter.hvd_adapter_set_timeline(h.h, int(timeline))
+        with torch.cuda.stream(side):
+            torch.cuda._sleep(60_000_000)  # tens of milliseconds; the kernel ends by itself
+            for t, f in zip(tensors, fresh):
+                t.copy_(f)
+            ready.record(side)
+        adapter.hvd_adapter_next_ready_events(h.h, _ptrs([ready.cuda_event]), 1)
+        rc, msg = h.allreduce([t.data_ptr() for t in tensors], [o.data_ptr() for o in outs], counts, F32, 0.5, 1.0)
+        assert rc == 0, msg
+        torch.cuda.synchronize()
+        for f, o in zip(fresh, outs):
+            want = orc.scale_buffer(f.cpu().numpy(), 0.5, F32)
+            assert np.array_equal(o.cpu().numpy().view(np.uint32), want.view(np.uint32))
+        if timeline:
+            out = ctypes.create_string_buffer(512)
+            adapter.hvd_adapter_timeline(h.h, out, 512)
+            assert out.value.decode().split(",")[0] == "WAIT_FOR_DATA"
+    finally:
+        h.close()
