@@ -506,3 +506,22 @@ def test_unpack_record_without_payload_records_the_event(gpu):
     horovod_amd.check(L.hvdhip_event_release(gpu.stream.handle, ev), "hvdhip_event_release")
     assert L.hvdhip_fusion_unpack_record(plan.handle, None, 1.0, gpu.stream.handle, None) == -1  # event is NULL
     plan.destroy()
+
+
+@pytest.mark.parametrize("nchunks", [1, 2, 7, 8, 9, 31, 32, 33, 63, 64, 65, 255, 256, 257, 511, 512, 513, 4095, 4096, 4097])
+def test_table_sizes_around_the_group_boundaries(gpu, orc, nchunks):
+    """Chunk tables are padded to a multiple of 32 entries and read through a mapping that permutes
+    entries within groups of 32 (and chunks within runs per XCD, in groups of 512): chunk counts on
+    both sides of every boundary, as one big tensor, as one-chunk tensors, and as a ragged mix, each
+    packed with a prescale and unpacked with a postscale, every byte inside and outside checked."""
+    per = 1024  # fp32 elements of a 4 KiB chunk
+    _check_round_trip(gpu, orc, [nchunks * per - 3], F32, 0.5, 0.25, seed=nchunks)
+    if nchunks <= 513:
+        _check_round_trip(gpu, orc, [per] * nchunks, F32, 0.5, 1.0, seed=nchunks + 1)
+        rng = np.random.default_rng(nchunks)
+        counts, left = [], nchunks
+        while left > 0:
+            k = int(min(left, rng.integers(1, 6)))
+            counts.append(k * per - int(rng.integers(0, per - 1)))
+            left -= k
+        _check_round_trip(gpu, orc, counts, F32, 1.0, 0.5, seed=nchunks + 2)
