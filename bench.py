@@ -23,6 +23,11 @@ rate of the roofline kernel).  `ms_per_step` is the wall-clock mean of the K tim
 The HBM claim is `roofline`: the dominant kernel of the workload launched back to back on rotating
 buffers, algorithmic bytes per launch over its launch time from HIP events on its stream (mean over
 ten batches of launches, with median / min / max of the batches), against the 8 TB/s peak.
+`roofline.traffic` (HBM bytes per launch) is measured in the same run: before it touches the GPU
+itself the benchmark starts four rocprofv3 child runs (FETCH_SIZE and WRITE_SIZE over the headline's
+kernel loops and over the calibration copies) and scales the counters; if that cannot be done
+(no rocprofv3, the run is itself under a profiler, `--no-live-traffic`) the figure of the committed
+profile stands in and `roofline.traffic_from` says so.
 `cpu_baseline` is the CPU oracle (a restatement of the reference's CPU path) on one host core over
 the same workload.  `extra` carries the other configurations: C1-C5 pipelines on one and two
 streams, C1 and C5 once more through the C++ adapter's GPUAllreduce::Execute with its finalizer
@@ -59,7 +64,8 @@ ROTATE = 6
 # WRITE_SIZE runs (KiB per dispatch), each scaled by what the same counter reads for two plain
 # 256 MiB device copies of known size that are not the library's own kernels
 # (`bench.py --calibrate`).  The summaries with the commands are the files named here under
-# profiles/; tests/test_host_logic.py re-derives every figure from them.
+# profiles/; tests/test_host_logic.py re-derives every figure from them.  A default run measures the
+# headline configuration's own figures again (live_traffic) and overwrites those entries.
 TRAFFIC_BYTES_MEASURED = {
     "ag.pack": 138114058,
     "ag.pack_small": 12592596,
@@ -126,6 +132,9 @@ def parse():
                          "library's kernel, by hipMemcpyAsync and by an elementwise kernel of torch, ag the allgather "
                          "fusion buffer's pack and unpack (8 ranks x 128 entries) at a 6 MB and at a 66 MB slab; "
                          "--steps launches per kernel after --warmup")
+    ap.add_argument("--no-live-traffic", action="store_true",
+                    help="take roofline.traffic from the committed profile instead of measuring it in this run with "
+                         "rocprofv3 child processes")
     ap.add_argument("--calibrate", action="store_true",
                     help="only launch a plain 256 MiB device copy (scales rocprofv3 byte counters)")
     return ap.parse_args()
@@ -1161,6 +1170,90 @@ def extras(headline_cases_block):
 
 
 # ----------------------------------------------------------------------------------------------
+# HBM traffic of the headline's kernels, measured in this run
+# ----------------------------------------------------------------------------------------------
+
+def _counter_rows(path):
+    import csv
+    csv.field_size_limit(1 << 30)
+    with open(path, newline="") as f:
+        rows = list(csv.DictReader(f))
+    rows.sort(key=lambda r: int(r["Start_Timestamp"]))
+    return rows
+
+
+def live_traffic(cfg="c1", launches=(2, 6), budget_s=240):
+    """HBM bytes per launch of every kernel loop of `cfg`, from rocprofv3 runs started by this process:
+    `bench.py --kernel-only cfg` under --pmc FETCH_SIZE and under --pmc WRITE_SIZE (KiB per dispatch),
+    each scaled by what the same counter reads for `bench.py --calibrate`, two plain 256 MiB copies that
+    are not the library's kernels.  Returns ({case: bytes}, note) or (None, why not).  Runs before this
+    process touches the GPU; any failure only means that the committed figures are reported instead."""
+    import glob
+    import shutil
+    import subprocess
+    import tempfile
+    if any(k.startswith("ROCPROF") or k.startswith("ROCP_") for k in os.environ):
+        return None, "this run is itself under a profiler"
+    if not shutil.which("rocprofv3"):
+        return None, "rocprofv3 is not on PATH"
+    warm, steps = launches
+    per = warm + steps
+    tmp = tempfile.mkdtemp(prefix="hvdhip_bench_", dir="/tmp")
+    t0 = time.time()
+    try:
+        def run(tag, counter, tail):
+            left = budget_s - (time.time() - t0)
+            if left < 20:
+                raise RuntimeError("out of time")
+            cmd = ["rocprofv3", "--pmc", counter, "--output-format", "csv", "-d", os.path.join(tmp, tag), "-o", "c", "--",
+                   sys.executable, os.path.join(ROOT, "bench.py")] + tail + ["--steps", str(steps), "--warmup", str(warm)]
+            r = subprocess.run(cmd, cwd=ROOT, env=dict(os.environ, TMPDIR="/tmp"), stdout=subprocess.PIPE,
+                               stderr=subprocess.DEVNULL, timeout=min(left, 120))
+            if r.returncode != 0:
+                raise RuntimeError("%s exited with %d" % (tag, r.returncode))
+            found = glob.glob(os.path.join(tmp, tag, "**", "*counter_collection.csv"), recursive=True)
+            if not found:
+                raise RuntimeError("%s wrote no counter file" % tag)
+            return r.stdout.decode(errors="replace"), _counter_rows(found[0])
+
+        factors = {}
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            _, rows = run("cal_" + counter, counter, ["--calibrate"])
+            seen = []
+            for frag in ("__amd_rocclr_copyBuffer", "vectorized_elementwise_kernel"):
+                v = [float(r["Counter_Value"]) for r in rows if frag in r["Kernel_Name"] and r["Counter_Name"] == counter][-per:]
+                if len(v) == per:
+                    seen.append(262144.0 * len(v) / sum(v))
+            if not seen or max(seen) / min(seen) > 1.01:
+                raise RuntimeError("calibration kernels disagree or are missing: %s" % seen)
+            factors[counter] = sum(seen) / len(seen)
+        totals = {}
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            out, rows = run(cfg + "_" + counter, counter, ["--kernel-only", cfg])
+            info = json.loads(next(l for l in out.splitlines() if l.startswith("CASES "))[6:])
+            lib = [r for r in rows if "hvdhip" in r["Kernel_Name"] and r["Counter_Name"] == counter]
+            need = sum(per * len(c["parts"]) for c in info["cases"])
+            if len(lib) < need:
+                raise RuntimeError("%d dispatches of the library's kernels, %d expected" % (len(lib), need))
+            lib = lib[len(lib) - need:]
+            at = 0
+            for c in info["cases"]:
+                n = per * len(c["parts"])
+                seg = lib[at + warm * len(c["parts"]):at + n]  # the warm-up launches lead
+                at += n
+                kib = sum(float(r["Counter_Value"]) for r in seg) / steps  # all kernels of one call together
+                totals[c["case"]] = totals.get(c["case"], 0.0) + kib * 1024 * factors[counter]
+        note = ("rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE child runs of `bench.py --kernel-only %s` in this run "
+                "(%d launches per kernel), scaled by the same counters over `bench.py --calibrate` (x %.4f, x %.4f)"
+                % (cfg, steps, factors["FETCH_SIZE"], factors["WRITE_SIZE"]))
+        return {k: int(round(v)) for k, v in totals.items()}, note
+    except Exception as e:  # the committed figures stand in
+        return None, "%s: %s" % (type(e).__name__, e)
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
+# ----------------------------------------------------------------------------------------------
 # output: one compact JSON line on stdout (it has to fit a reader's 8 KB window), everything on stderr
 # ----------------------------------------------------------------------------------------------
 
@@ -1216,6 +1309,12 @@ def main():
         print("bench.py measures one GPU's share of the hot path: this build has no inter-GPU collectives, "
               "run it with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    # The counter runs come first: child processes are started before this one has touched the GPU.
+    measured, traffic_note = None, None
+    if not (args.kernel_only or args.calibrate or args.no_live_traffic):
+        measured, traffic_note = live_traffic("c1")
+        if measured:
+            TRAFFIC_BYTES_MEASURED.update(measured)
     import torch
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -1293,6 +1392,8 @@ def main():
     roofline = dict(next(b for b in blocks if b["case"] == "c1.reduce"))
     roofline.pop("timed", None)
     roofline["why_this_kernel"] = "the reduce-sum takes the largest share of the pipeline's kernel time (3C of 7P bytes)"
+    roofline["traffic_from"] = traffic_note if measured else (
+        "the committed summary %s (not measured in this run: %s)" % (TRAFFIC_PROFILE["c1"], traffic_note or "--no-live-traffic"))
 
     result = {
         "metric": "achieved HBM GB/s (% of 8 TB/s) for fused pack+scale+reduce+unpack; Adasum GB/s",
