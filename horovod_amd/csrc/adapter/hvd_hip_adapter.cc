@@ -451,9 +451,24 @@ void GPUAllreduce::WaitForData(std::vector<TensorTableEntry>& entries) {
 
 Status GPUAllreduce::Execute(std::vector<TensorTableEntry>& entries, double prescale_factor,
                              double postscale_factor, const std::vector<const void*>& peers) {
-  auto& first_entry = entries[0];
   gpu_op_context_.InitGPU(entries);
   gpu_op_context_.InitGPUQueue(entries);
+  try {
+    return Queue(entries, prescale_factor, postscale_factor, peers);
+  } catch (...) {
+    // the op failed while it was being queued (the caller reports it, common/operations.cc:291-305):
+    // the events taken for it so far go back to their pool
+    try {
+      gpu_context_->ClearEvents(gpu_op_context_.event_queue);
+    } catch (const std::exception&) {
+    }
+    throw;
+  }
+}
+
+Status GPUAllreduce::Queue(std::vector<TensorTableEntry>& entries, double prescale_factor,
+                           double postscale_factor, const std::vector<const void*>& peers) {
+  auto& first_entry = entries[0];
   WaitForData(entries);
   const void* fused_input_data;
   void* buffer_data;

@@ -254,6 +254,9 @@ public:
   size_t cached_plans() const { return plans_.size(); }
 
 private:
+  // Execute after InitGPU / InitGPUQueue: everything from WaitForData to FinalizeGPUQueue.
+  Status Queue(std::vector<TensorTableEntry>& entries, double prescale_factor, double postscale_factor,
+               const std::vector<const void*>& peers);
   // Fused tensor sets repeat every step (the reference caches responses,
   // common/response_cache.cc:126-235): one resident plan per distinct entry list.
   hvdhip_fusion_plan* PlanFor(const std::vector<TensorTableEntry>& entries);

@@ -8,6 +8,7 @@
 #include <cstdlib>
 #include <mutex>
 #include <set>
+#include <stdexcept>
 #include <thread>
 #include <vector>
 
@@ -213,6 +214,25 @@ void failure_reaches_callbacks() {
   std::printf("failure: %s\n", r.reason.c_str());
 }
 
+// 3b. A response that fails while it is being queued (an unsupported dtype reaches the pack) throws out
+//     of Execute, calls no callback, and leaves no pooled event behind.
+void failure_while_queueing() {
+  Rig rig(1, 1, false, false, /*timeline=*/true);  // the QUEUE event is already in the op's queue when the pack fails
+  const std::vector<int> counts = {10, 20};
+  Response r;
+  build(r, 11, counts);
+  for (auto& e : r.entries) e.dtype = HOROVOD_INT32;  // the pretend device packs float32 only
+  bool threw = false;
+  try {
+    rig.op->Execute(r.entries, 1.0, 1.0, {});
+  } catch (const std::logic_error&) {
+    threw = true;
+  }
+  rig.context.finalizer_thread_pool.wait_idle();
+  REQUIRE(threw && r.callbacks == 0);
+  REQUIRE(fake_events_outstanding() == 0);
+}
+
 // 4. No finalizer threads: the completion runs on the caller's thread before Execute returns.
 void inline_completion() {
   Rig rig(2, 0);
@@ -333,6 +353,7 @@ int main() {
   many_responses();
   two_in_flight();
   failure_reaches_callbacks();
+  failure_while_queueing();
   inline_completion();
   async_completion();
   elastic_and_timeline();
