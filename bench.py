@@ -784,9 +784,7 @@ def cpu_baseline_resnet(budget_s=12.0):
     gbs = 7 * 4 * n * reps / dt / 1e9
     return {"value": round(gbs, 3), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": "%d passes over the whole 161-tensor set (memcpy pack, in-place ScaleBuffer 0.125, sum with one "
-                      "peer buffer, memcpy unpack; 7P algorithmic bytes each, one buffer for all tensors as the CPU "
-                      "path has no 64 MiB cycles to gain from) in %.1f s; host has %d cores"
-                      % (reps, dt, os.cpu_count())}
+                      "peer buffer, memcpy unpack; 7P bytes each) in %.1f s; host has %d cores" % (reps, dt, os.cpu_count())}
 
 
 def cpu_extras(budget_s=2.5):
@@ -1243,8 +1241,8 @@ def live_traffic(cfg="c1", launches=(2, 6), budget_s=240):
                 at += n
                 kib = sum(float(r["Counter_Value"]) for r in seg) / steps  # all kernels of one call together
                 totals[c["case"]] = totals.get(c["case"], 0.0) + kib * 1024 * factors[counter]
-        note = ("rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE child runs of `bench.py --kernel-only %s` in this run "
-                "(%d launches per kernel), scaled by the same counters over `bench.py --calibrate` (x %.4f, x %.4f)"
+        note = ("this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over `bench.py --kernel-only %s` (%d launches), scaled by "
+                "the same counters over `bench.py --calibrate` (x %.4f, x %.4f)"
                 % (cfg, steps, factors["FETCH_SIZE"], factors["WRITE_SIZE"]))
         return {k: int(round(v)) for k, v in totals.items()}, note
     except Exception as e:  # the committed figures stand in
@@ -1257,15 +1255,16 @@ def live_traffic(cfg="c1", launches=(2, 6), budget_s=240):
 # output: one compact JSON line on stdout (it has to fit a reader's 8 KB window), everything on stderr
 # ----------------------------------------------------------------------------------------------
 
-KERNEL_COLUMNS = ["case", "kernel", "launch_us", "us_median", "us_min", "us_max", "frac_of_8TBps",
-                  "algorithmic_B", "traffic_B", "in_pipeline_us"]
+# (a case's kernel is named in the profile that `case` leads to -- profiles/<config>_*_kernels.txt -- and on stderr)
+KERNEL_COLUMNS = ["case", "launch_us", "us_median", "us_min", "us_max", "frac_of_8TBps", "algorithmic_B", "traffic_B",
+                  "in_pipeline_us"]
 PIPELINE_COLUMNS = ["algorithmic_GB/s", "frac_of_8TBps", "ms", "ms_median", "ms_min", "ms_max", "streams", "cpu_GB/s_1core"]
 
 
 def kernel_row(b):
     m = b.get("launch_us_median_min_max") or [None, None, None]
-    return [b["case"], b["kernel"], b["launch_us"], m[0], m[1], m[2], b["frac"], b["algorithmic_bytes_per_launch"],
-            b.get("traffic"), b.get("in_pipeline_us")]
+    return [b["case"], b["launch_us"], m[0], m[1], m[2], b["frac"], b["algorithmic_bytes_per_launch"], b.get("traffic"),
+            b.get("in_pipeline_us")]
 
 
 def compact(result):
@@ -1401,12 +1400,12 @@ def main():
         "ms_per_step": round(sec * 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic", "config": config,
         # `value` counts algorithmic bytes over wall time; these three name what is what
-        "value_kind": "algorithmic GB/s of the whole pipeline (buffer hand-overs through the Infinity Cache included)",
+        "value_kind": "algorithmic GB/s of the whole pipeline (hand-overs through the Infinity Cache included)",
         "hbm_GB/s": round(roofline["traffic"] / (roofline["launch_us"] * 1e-6) / 1e9, 1) if roofline.get("traffic") else None,
-        "hbm_GB/s_is": "counter-derived HBM bytes per launch of the roofline kernel (profiles/) / its launch time in this run",
+        "hbm_GB/s_is": "roofline.traffic / the roofline kernel's launch time",
         "algorithmic_frac_of_8TBps": round(value / HBM_PEAK_GBS, 4),
         "ms_per_step_median_min_max": spread(each, 1e3, 5),
-        "ms_per_step_from": "HIP event pair around each of the %d timed steps, on the pipeline's stream" % args.steps,
+        "ms_per_step_from": "a HIP event pair around each timed step",
         "roofline": roofline,
         "traffic_profile": TRAFFIC_PROFILE["c1"],
     }

@@ -114,3 +114,74 @@ def test_traffic_constants_of_the_bench_follow_from_the_profiles():
                 in_pipeline[pair[0].split(".")[0] + "." + pair[1]] = float(r["avg_ns"])
     assert seen == bench.TRAFFIC_BYTES_MEASURED
     assert in_pipeline == bench.IN_PIPELINE_NS_MEASURED
+
+
+def _bench():
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_module", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    return bench
+
+
+def test_spread_is_median_min_max():
+    bench = _bench()
+    assert bench.spread([3.0, 1.0, 2.0]) == [2.0, 1.0, 3.0]
+    assert bench.spread([4.0, 1.0, 2.0, 3.0]) == [2.5, 1.0, 4.0]
+    assert bench.spread([0.001234567], scale=1e3, digits=3) == [1.235, 1.235, 1.235]
+
+
+def test_the_stdout_line_stays_inside_a_readers_window():
+    """bench.py prints one JSON line that a reader who keeps the last 8 KB must see whole: built here
+    from a result of the shape a full run produces (every pipeline and kernel loop the benchmark has,
+    with realistic figures), the compact line has every contract key and stays under 8,000 bytes."""
+    import json
+    bench = _bench()
+    block = {"bound": "hbm", "kernel": "reduce_k<_Float16, 7, 1> + xfer_k<Copy<unsigned short>, 1, 0>", "case": "c1.pack_rotating_destination",
+             "launch_us": 123.45, "launch_us_median_min_max": [123.45, 122.22, 125.67], "timed_batches": 10,
+             "algorithmic_bytes_per_launch": 2147483648, "achieved": 6543.2, "peak": 8000.0, "unit": "GB/s", "frac": 0.8179,
+             "traffic": 2164248147, "workgroups": 262144, "timed": "x" * 300, "in_pipeline_us": 18.11}
+    pipe = {"algorithmic_GB/s": 6543.2, "algorithmic_frac_of_8TBps": 0.8179, "ms": 3.1453, "ms_median_min_max": [3.1481, 3.1155, 3.1734],
+            "algorithmic_MB": 21468.2, "cycles": 49, "streams": 2, "peers": 1, "reduce": "k-way", "cpu_GB/s": 52.04,
+            "completion_event_per_cycle": True, "replicas_rotated": 1, "note": "y" * 400, "vs_python_pipeline": 0.9956}
+    names = ["c1_resnet50_fp32_one_stream", "c1_resnet50_fp32_one_slot_through_the_adapter", "c1_resnet50_fp32_two_streams",
+             "c1_resnet50_fp32_one_stream_completion_events", "c2_fusion_stress", "c2_fusion_stress_one_stream_completion_events",
+             "c2_fusion_stress_one_stream_completion_events_with_unpack", "c2_fusion_stress_two_streams",
+             "c2_fusion_stress_two_streams_no_completion_events", "c3_bert_large_fp32_to_fp16_7peers_eighth_share",
+             "c3_bert_large_postscale_4", "c3_bert_large_two_streams", "c4_adasum_fp32_2x32M_64layers", "c4_adasum_fp16_2x32M_64layers",
+             "c5_gpt2_xl_fp16_two_streams", "c5_gpt2_xl_fp16_two_slots_through_the_adapter", "c5_gpt2_xl_fp16_one_stream",
+             "c5_gpt2_xl_fp16_array_entry_points", "allgather_fusion_8ranks_128entries_6MB_slab",
+             "allgather_fusion_8ranks_128entries_66MB_slab"]
+    extra = {}
+    k = 0
+    for i, n in enumerate(names):
+        extra[n] = dict(pipe)
+        if i % 4 == 0:  # 30 kernel loops in all, as a full run has
+            extra[n]["kernels"] = []
+            for _ in range(6):
+                b = dict(block)
+                b["case"] = "c%d.unpack_postscale%02d" % (i % 5 + 1, k)
+                k += 1
+                extra[n]["kernels"].append(b)
+    extra["c2_fusion_stress"]["execute_vs_per_tensor_copies"] = {"offset_table_kernels_ms": 0.075, "per_tensor_copies_ms": 4.7525, "speedup": 63.4}
+    roofline = dict(block, why_this_kernel="z" * 90, traffic_from="w" * 200)
+    roofline.pop("timed")
+    result = {"metric": "achieved HBM GB/s (% of 8 TB/s) for fused pack+scale+reduce+unpack; Adasum GB/s", "value": 6716.0, "unit": "GB/s",
+              "n_gpus": 1, "steps": 20, "warmup": 5, "ms_per_step": 5.32758, "higher_is_better": True, "scaling": "weak",
+              "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+              "config": {"workload": "v" * 340, "tensors": 161, "payload_bytes": 102228128, "cycles": 2,
+                         "cycle_buffer_bytes": [62529792, 39698432], "fusion_threshold": 67108864, "peers": 1, "prescale": 0.125,
+                         "postscale": 1.0, "passes_per_step": 50, "algorithmic_bytes_per_step": 35779845000, "replicas_rotated": 4,
+                         "streams": 1, "value_is": "u" * 300},
+              "value_kind": "t" * 100, "hbm_GB/s": 6295.3, "hbm_GB/s_is": "s" * 55, "algorithmic_frac_of_8TBps": 0.8395,
+              "ms_per_step_median_min_max": [5.32095, 5.31297, 5.32813], "ms_per_step_from": "r" * 40, "roofline": roofline,
+              "traffic_profile": "profiles/c1_resnet50_fp32_kernels.txt",
+              "cpu_baseline": {"value": 53.094, "unit": "GB/s", "cores": 1, "kind": "port", "sample": "q" * 210}, "extra": extra}
+    line = json.dumps(bench.compact(result), separators=(",", ":"))
+    assert len(line) < 7400, len(line)  # a margin for names and notes that grow
+    back = json.loads(line)
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in back
+    assert len(back["extra"]["pipelines"]) == len(names) and len(back["extra"]["kernels"]) == 30
+    assert back["extra"]["kernel_columns"][0] == "case" and len(back["extra"]["kernels"][0]) == len(back["extra"]["kernel_columns"])
