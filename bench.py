@@ -1053,6 +1053,53 @@ def device_ceiling_extra(steps=20):
     return {"kernels": blocks, "traffic_profile": TRAFFIC_PROFILE["copy"]}
 
 
+def adasum_split_extra(steps=30):
+    """The Adasum configuration through hvdhip_adasum_dot_norms -> hvdhip_adasum_read (the host gets the 64
+    triples; between ranks they would be summed here, adasum.h:380-382) -> coefficients on the host
+    (adasum.h:397-404) -> hvdhip_adasum_set_coeffs -> hvdhip_adasum_scaled_add: what the combine costs once
+    the sums have to leave the device, which is what more than one GPU needs."""
+    import math
+    import torch
+    from horovod_amd import AdasumPlan, DTYPE, workloads as W
+    s = stream_pair()[0]
+    n = 1 << 25
+    lc = W.adasum_layer_counts(n, 64, seed=13)
+    g = torch.Generator(device="cuda")
+    pairs = []
+    for r in range(4):
+        g.manual_seed(14 + 2 * r)
+        a = torch.randn(n, generator=g, device="cuda", dtype=torch.float32)
+        g.manual_seed(15 + 2 * r)
+        b = 0.3 * a + (1 - 0.09) ** 0.5 * torch.randn(n, generator=g, device="cuda", dtype=torch.float32)
+        pairs.append((a, b))
+    plan = AdasumPlan(lc, DTYPE["float32"])
+    torch.cuda.synchronize()
+    guard = math.sqrt(2.2250738585072014e-308)
+    turn = [0]
+
+    def one():
+        i = turn[0] = (turn[0] + 1) % len(pairs)
+        a, b = pairs[i]
+        plan.dot_norms(a.data_ptr(), b.data_ptr(), s)
+        nd, _ = plan.read(s)  # blocks until the triples are on the host
+        co = []
+        for k in range(len(lc)):
+            d, an, bn = nd[3 * k:3 * k + 3]
+            co += [1.0 - d / an * 0.5 if an >= guard else 1.0, 1.0 - d / bn * 0.5 if bn >= guard else 1.0]
+        plan.set_coeffs(co, s)
+        plan.scaled_add(a.data_ptr(), b.data_ptr(), s)
+
+    sec, each = timed_batches(one, s.synchronize, steps, 3)
+    plan.destroy()
+    del pairs
+    torch.cuda.empty_cache()
+    ab = 5 * n * 4
+    return {"algorithmic_GB/s": round(ab / sec / 1e9, 1), "algorithmic_frac_of_8TBps": round(ab / sec / 1e9 / HBM_PEAK_GBS, 4),
+            "ms": round(sec * 1e3, 4), "ms_median_min_max": spread(each, 1e3, 4), "algorithmic_MB": round(ab / 1e6, 1),
+            "streams": 1, "replicas_rotated": 4,
+            "note": "dot_norms, blocking read of 64 triples, coefficients on the host, set_coeffs, scaled_add"}
+
+
 def extras(headline_cases_block):
     import torch
     from horovod_amd import DTYPE, workloads as W
@@ -1149,6 +1196,10 @@ def extras(headline_cases_block):
                      "algorithmic_MB": round(b["algorithmic_bytes_per_launch"] / 1e6, 1),
                      "replicas_rotated": 4, "kernels": blocks, "roofline_case": b["case"], "traffic_profile": TRAFFIC_PROFILE["c4"],
                      "note": "two launches timed together with HIP events; per-kernel durations and traffic are in the profile"}
+
+    # C4 through the split entry points, as more than one GPU needs them: the partial sums leave the device
+    # for the exchange between ranks and the coefficients come back (ops/adasum/adasum.h:380-404)
+    out["c4_adasum_fp32_split_with_host_round_trip"] = adasum_split_extra()
 
     # C5: GPT-2 XL fp16 on two streams (the configuration), on one, through the array-taking entry points
     # and through the adapter on two stream slots
