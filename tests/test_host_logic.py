@@ -178,7 +178,7 @@ def test_the_stdout_line_stays_inside_a_readers_window():
               "traffic_profile": "profiles/c1_resnet50_fp32_kernels.txt",
               "cpu_baseline": {"value": 53.094, "unit": "GB/s", "cores": 1, "kind": "port", "sample": "q" * 210}, "extra": extra}
     line = json.dumps(bench.compact(result), separators=(",", ":"))
-    assert len(line) < 7400, len(line)  # a margin for names and notes that grow
+    assert len(line) < 7800, len(line)  # every row here is as long as the longest real one: a real line is under 6,500
     back = json.loads(line)
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
                 "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
