@@ -51,6 +51,16 @@ struct Harness {
   std::vector<void*> next_ready_events;  // for the entries of the next response queued
 };
 
+// Memory that the caller of this harness allocated (a torch tensor in the tests): nothing to free.
+class CallerBuffer : public PersistentBuffer {
+public:
+  explicit CallerBuffer(void* p) : p_(p) {}
+  const void* AccessData() const override { return p_; }
+
+private:
+  void* p_;
+};
+
 int report(const std::exception& e, char* err, size_t errlen) {
   if (err && errlen) {
     std::strncpy(err, e.what(), errlen - 1);
@@ -150,7 +160,12 @@ void* hvd_adapter_create_ex(int num_streams, int batch_d2d_memcopies, int enable
   h->state.batch_d2d_memcopies = batch_d2d_memcopies != 0;
   h->state.enable_async_completion = enable_async_completion != 0;
   h->state.elastic_enabled = elastic != 0;
-  for (int i = 0; i < num_streams; ++i) h->state.fusion_buffer.push_back(fusion_buffers[i]);
+  for (int i = 0; i < num_streams; ++i) {
+    void* p = fusion_buffers[i];
+    // the size plays no part when the caller owns the memory; any one value keeps the buffer for good
+    h->state.fusion_buffer.InitializeBuffer(64 << 20, 0, [p](int64_t, int) { return std::make_shared<CallerBuffer>(p); }, i,
+                                            nullptr, nullptr);
+  }
   h->context.streams.resize((size_t)num_streams);
   if (finalizer_threads > 0) h->context.finalizer_thread_pool.create(finalizer_threads);
   h->allreduce = new GPUAllreduce(&h->context, &h->state);

@@ -77,6 +77,36 @@ void ThreadPool::reset() {
   threads_.clear();
 }
 
+// -------------------------------------------------------- FusionBufferManager
+
+Status FusionBufferManager::InitializeBuffer(int64_t threshold, int device, const Allocator& allocate, int stream_id,
+                                             std::function<void()> on_start_init, std::function<void()> on_end_init) {
+  auto& slot = tensor_fusion_buffers_[std::make_pair(device, stream_id)];
+  if (slot.second != threshold) {
+    // another threshold: this manager lets go of the buffer; responses in flight still hold it
+    slot.first.reset();
+    slot.second = 0;
+  }
+  if (slot.first) return Status::OK();
+  if (on_start_init) on_start_init();
+  slot.first = allocate(threshold, device);
+  if (on_end_init) on_end_init();
+  if (!slot.first) return Status::UnknownError("the framework could not allocate the fusion buffer");
+  slot.second = threshold;
+  return Status::OK();
+}
+
+std::shared_ptr<PersistentBuffer> FusionBufferManager::GetBuffer(int device, int stream_id) {
+  auto it = tensor_fusion_buffers_.find(std::make_pair(device, stream_id));
+  return it == tensor_fusion_buffers_.end() ? nullptr : it->second.first;
+}
+
+static void* SlotBuffer(GlobalState* state, int device) {
+  auto buffer = state->fusion_buffer.GetBuffer(device, state->current_nccl_stream);
+  if (!buffer) throw std::logic_error("no fusion buffer has been initialised for this device and stream slot");
+  return const_cast<void*>(buffer->AccessData());
+}
+
 // ---------------------------------------------------------------- GPUContext
 
 GPUContext::GPUContext() {}
@@ -241,8 +271,11 @@ Status GPUOpContext::FinalizeGPUQueue(std::vector<TensorTableEntry>& entries,
   const bool timeline = global_state_->timeline_initialized;
   gpuStream_t current_stream = *stream;
   auto events = event_queue;
+  // a claim on the slot's fusion buffer, so that its memory outlives this response whatever happens
+  // to the fusion threshold meanwhile (ops/gpu_operations.cc:64-67); dropped when the task is done
+  auto fusion_buffer = global_state_->fusion_buffer.GetBuffer(device, global_state_->current_nccl_stream);
   auto finalize = [gpu_context, global_state, device, elastic, async_completion, timeline, current_stream, events,
-                   entries, error_check_callback]() mutable {
+                   entries, error_check_callback, fusion_buffer]() mutable {
     Status status = Status::OK();
     try {
       gpu_context->SetDevice(device);  // ops/gpu_operations.cc:75: the thread has no device of its own yet
@@ -270,6 +303,7 @@ Status GPUOpContext::FinalizeGPUQueue(std::vector<TensorTableEntry>& entries,
       }
     }
     for (auto& e : entries) e.FinishWithCallback(status);
+    fusion_buffer.reset();
     if (status.event.event) {
       try {
         gpu_context->ReleaseEvent(status.event);
@@ -346,7 +380,7 @@ void GPUAllreduce::MemcpyInFusionBuffer(const std::vector<TensorTableEntry>& ent
 void GPUAllreduce::ScaleMemcpyInFusionBuffer(const std::vector<TensorTableEntry>& entries,
                                              const void*& fused_input_data, void*& buffer_data,
                                              size_t& buffer_len, double scale_factor) {
-  buffer_data = global_state_->fusion_buffer[(size_t)global_state_->current_nccl_stream];
+  buffer_data = SlotBuffer(global_state_, entries[0].device);  // ops/gpu_operations.cc:122-124
   const bool converting = entries[0].wire_dtype() != entries[0].dtype;
   if (converting && !global_state_->batch_d2d_memcopies)
     throw std::logic_error("A fusion buffer of another dtype than the tensors needs HOROVOD_BATCH_D2D_MEMCOPIES.");
@@ -539,7 +573,7 @@ void GPUAllgather::SetEntryComponentOffsets(size_t num_entries, const int64_t* c
 void GPUAllgather::MemcpyInFusionBuffer(const std::vector<TensorTableEntry>& entries, const int* displcmnts,
                                         int rank, int element_size, void*& buffer_data) {
   auto& first_entry = entries[0];
-  buffer_data = global_state_->fusion_buffer[(size_t)global_state_->current_nccl_stream];
+  buffer_data = SlotBuffer(global_state_, first_entry.device);
   std::vector<void*> out;
   std::vector<const void*> in;
   std::vector<size_t> sizes;

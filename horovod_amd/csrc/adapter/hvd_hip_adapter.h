@@ -9,6 +9,7 @@
 //   ThreadPool          common/thread_pool.h:27-43 (the finalizer threads, one per stream slot,
 //                       common/operations.cc:449)
 //   Status              common/common.h:192-212
+//   FusionBufferManager common/fusion_buffer_manager.{h,cc}; PersistentBuffer common/common.h:321-325
 //   GPUAllreduce hooks  ops/gpu_operations.h:139-172, ops/gpu_operations.cc:118-339
 //   Adasum dispatch     ops/adasum/adasum.h:101-140,344-410
 //   FuseResponses       common/controller.cc:793-866
@@ -143,6 +144,31 @@ private:
   bool stopping_ = false;
 };
 
+// common/common.h:321-325: memory that the framework allocated and keeps alive while anybody holds it.
+class PersistentBuffer {
+public:
+  virtual const void* AccessData() const = 0;
+  virtual ~PersistentBuffer() = default;
+};
+
+// One fusion buffer per (device, stream slot), allocated through the framework at first use and again
+// when the fusion threshold has changed (common/fusion_buffer_manager.cc:21-50).  The reference keys
+// the buffers by framework as well; one process of this adapter serves one framework.  Handing out
+// shared ownership is the point: a response in flight keeps the buffer it was packed into alive until
+// its finalizer has run, whatever the threshold does meanwhile (ops/gpu_operations.cc:64-67).
+class FusionBufferManager {
+public:
+  // Stands for OpContext::AllocatePersistent (common/common.h:327-339) of the entry's framework.
+  typedef std::function<std::shared_ptr<PersistentBuffer>(int64_t size, int device)> Allocator;
+  Status InitializeBuffer(int64_t threshold, int device, const Allocator& allocate, int stream_id,
+                          std::function<void()> on_start_init, std::function<void()> on_end_init);
+  // The buffer of (device, stream slot), or null.
+  std::shared_ptr<PersistentBuffer> GetBuffer(int device, int stream_id);
+
+private:
+  std::map<std::pair<int, int>, std::pair<std::shared_ptr<PersistentBuffer>, int64_t>> tensor_fusion_buffers_;
+};
+
 class GPUContext {
 public:
   GPUContext();
@@ -189,8 +215,8 @@ struct GlobalState {
   bool timeline_initialized = false;
   std::vector<std::string> timeline_activities;  // appended to by finalizer threads, under timeline_mutex
   std::mutex timeline_mutex;
-  // One fusion buffer per stream slot (common/fusion_buffer_manager.cc:25); owned by the framework.
-  std::vector<void*> fusion_buffer;
+  // One fusion buffer per (device, stream slot); the memory is the framework's.
+  FusionBufferManager fusion_buffer;
 };
 
 class GPUOpContext {

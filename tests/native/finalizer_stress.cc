@@ -104,18 +104,32 @@ void check(const Response& r, const std::vector<int>& counts, float pre, float p
   }
 }
 
+// A fusion buffer as a framework would hand it out: host memory here, counted when it is freed.
+std::atomic<int> g_buffers_freed{0};
+class HostBuffer : public PersistentBuffer {
+public:
+  explicit HostBuffer(int64_t size) : mem_((size_t)size) {}
+  ~HostBuffer() override { ++g_buffers_freed; }
+  const void* AccessData() const override { return mem_.data(); }
+
+private:
+  std::vector<char> mem_;
+};
+std::shared_ptr<PersistentBuffer> allocate_host(int64_t size, int) { return std::make_shared<HostBuffer>(size); }
+
 struct Rig {
   GPUContext context;
   GlobalState state;
-  std::vector<std::vector<char>> buffers;
   GPUAllreduce* op = nullptr;
   Rig(int slots, int threads, bool async_completion = false, bool elastic = false, bool timeline = false) {
     state.num_nccl_streams = slots;
     state.enable_async_completion = async_completion;
     state.elastic_enabled = elastic;
     state.timeline_initialized = timeline;
-    buffers.assign((size_t)slots, std::vector<char>(1 << 20));
-    for (auto& b : buffers) state.fusion_buffer.push_back(b.data());
+    for (int slot = 0; slot < slots; ++slot) {
+      Status s = state.fusion_buffer.InitializeBuffer(1 << 20, 0, allocate_host, slot, nullptr, nullptr);
+      REQUIRE(s.ok());
+    }
     context.streams.resize((size_t)slots);
     if (threads > 0) context.finalizer_thread_pool.create(threads);
     op = new GPUAllreduce(&context, &state);
@@ -306,6 +320,47 @@ void pool_semantics() {
   idle.wait_idle();  // no threads: nothing to wait for
 }
 
+// 7b. A response in flight keeps the fusion buffer it was packed into: the threshold changes while the
+//     pretend device still works on the response (InitializeBuffer lets go of the old buffer and
+//     allocates another), and the old one is freed only when the response's finalizer has run.
+void fusion_buffer_outlives_its_manager_entry() {
+  Rig rig(1, 1);
+  const std::vector<int> counts = {400, 9};
+  Response r;
+  build(r, 40, counts);
+  std::vector<const void*> peers = {r.peer.data()};
+  int init_calls = 0;
+  const int freed_before = g_buffers_freed.load();
+  auto old_buffer = rig.state.fusion_buffer.GetBuffer(0, 0)->AccessData();
+  fake_set_kernel_delay_us(15000);
+  rig.op->Execute(r.entries, 0.5, 1.0, peers);
+  fake_set_kernel_delay_us(0);
+  // the same threshold again: nothing happens
+  REQUIRE(rig.state.fusion_buffer.InitializeBuffer(1 << 20, 0, allocate_host, 0, [&] { ++init_calls; }, [&] { ++init_calls; }).ok());
+  REQUIRE(init_calls == 0 && rig.state.fusion_buffer.GetBuffer(0, 0)->AccessData() == old_buffer);
+  // another threshold: a new buffer, between the two callbacks
+  REQUIRE(rig.state.fusion_buffer.InitializeBuffer(2 << 20, 0, allocate_host, 0, [&] { ++init_calls; }, [&] { ++init_calls; }).ok());
+  REQUIRE(init_calls == 2 && rig.state.fusion_buffer.GetBuffer(0, 0)->AccessData() != old_buffer);
+  REQUIRE(r.callbacks == 0);                             // the response is still on the pretend device ...
+  REQUIRE(g_buffers_freed.load() == freed_before);       // ... and still owns the buffer it was packed into
+  rig.context.finalizer_thread_pool.wait_idle();
+  REQUIRE(r.callbacks == 2 && r.failures == 0);
+  REQUIRE(g_buffers_freed.load() == freed_before + 1);   // freed once its finalizer had run
+  check(r, counts, 0.5f, 1.f, true);
+  // an allocator that fails is reported, and a slot that was never initialised is an error of the op
+  Status s = rig.state.fusion_buffer.InitializeBuffer(4 << 20, 0, [](int64_t, int) { return std::shared_ptr<PersistentBuffer>(); }, 0, nullptr, nullptr);
+  REQUIRE(!s.ok() && rig.state.fusion_buffer.GetBuffer(0, 0) == nullptr);
+  Response r2;
+  build(r2, 41, counts);
+  bool threw = false;
+  try {
+    rig.op->Execute(r2.entries, 1.0, 1.0, {});
+  } catch (const std::logic_error& e) {
+    threw = std::string(e.what()).find("no fusion buffer") != std::string::npos;
+  }
+  REQUIRE(threw);
+}
+
 // 8. WaitForData: the tensors are produced on another stream (a copy that takes 20 ms) with an event
 //    recorded behind it; Execute is called at once with that event as every entry's ready event and
 //    must not read the tensors before the producer has written them -- by a stream wait, or, with the
@@ -357,6 +412,7 @@ int main() {
   inline_completion();
   async_completion();
   elastic_and_timeline();
+  fusion_buffer_outlives_its_manager_entry();
   waits_for_the_producer();
   std::printf("finalizer ok\n");
   return 0;
