@@ -53,6 +53,7 @@ std::size_t DataType_Size(DataType value);            // common/message.cc:66-92
 const std::string& DataType_Name(DataType value);     // common/message.cc:40-64
 
 typedef void* gpuStream_t;
+#define CPU_DEVICE_ID (-1)  // common/common.h:150
 
 // Activity names of the stages on this path, common/common.h:73-105.
 #define WAIT_FOR_DATA "WAIT_FOR_DATA"
@@ -250,6 +251,9 @@ class GPUAllreduce {
 public:
   GPUAllreduce(GPUContext* context, GlobalState* global_state);
   ~GPUAllreduce();
+
+  // ops/gpu_operations.cc:110-115: this op takes the response when its tensors live on a GPU.
+  bool Enabled(const std::vector<TensorTableEntry>& entries) const { return entries[0].device != CPU_DEVICE_ID; }
 
   // The op sequence of NCCLAllreduce::Execute (ops/nccl_operations.cc:156-214) with the
   // collective replaced by a local sum with `peers` (device buffers laid out like the
