@@ -400,6 +400,65 @@ void waits_for_the_producer() {
   }
 }
 
+// 9. The allgather op's fusion-buffer hooks (ops/collective_operations.cc:200-275): every rank's entries
+//    packed at the rank's displacement, then one component per (entry, rank) copied out; ragged first
+//    dimensions, an empty component.  Each output must be the ranks' tensors one after the other.
+void allgather_hooks() {
+  Rig rig(1, 1);
+  GPUAllgather op(&rig.context, &rig.state);
+  const int ranks = 3, n = 4;
+  const int64_t sizes[n][ranks] = {{5, 0, 7}, {100, 3, 1}, {1, 1, 1}, {33, 64, 2}};  // elements of entry e on rank r
+  std::vector<std::vector<std::vector<float>>> tensors((size_t)ranks);   // [rank][entry]
+  std::vector<std::vector<float>> outputs((size_t)n);
+  std::vector<int> recvcounts((size_t)ranks, 0), displ((size_t)ranks, 0);
+  std::vector<std::vector<int64_t>> csz((size_t)n, std::vector<int64_t>((size_t)ranks)), cof = csz;
+  std::vector<int64_t*> csz_p, cof_p;
+  float next = 1.f;
+  for (int r = 0; r < ranks; ++r) {
+    tensors[(size_t)r].resize((size_t)n);
+    for (int e = 0; e < n; ++e) {
+      for (int64_t i = 0; i < sizes[e][r]; ++i) tensors[(size_t)r][(size_t)e].push_back(next++);
+      recvcounts[(size_t)r] += (int)sizes[e][r];
+    }
+  }
+  for (int e = 0; e < n; ++e) {
+    int64_t total = 0;
+    for (int r = 0; r < ranks; ++r) {
+      csz[(size_t)e][(size_t)r] = sizes[e][r];
+      total += sizes[e][r];
+    }
+    outputs[(size_t)e].assign((size_t)total, -1.f);
+    csz_p.push_back(csz[(size_t)e].data());
+    cof_p.push_back(cof[(size_t)e].data());
+  }
+  int* dp = displ.data();
+  GPUAllgather::SetDisplacements(recvcounts.data(), dp, ranks);
+  REQUIRE(displ[0] == 0 && displ[1] == recvcounts[0] && displ[2] == recvcounts[0] + recvcounts[1]);
+  int64_t** cofpp = cof_p.data();
+  GPUAllgather::SetEntryComponentOffsets((size_t)n, csz_p.data(), recvcounts.data(), cofpp, ranks);
+  REQUIRE(hvdhip_set_device(0) == 0);
+  rig.context.StreamCreate(&rig.context.streams[0][0]);
+  void* buffer_data = nullptr;
+  std::vector<TensorTableEntry> entries((size_t)n);
+  for (int r = 0; r < ranks; ++r) {
+    for (int e = 0; e < n; ++e) {
+      entries[(size_t)e].tensor_data = tensors[(size_t)r][(size_t)e].data();
+      entries[(size_t)e].output_data = outputs[(size_t)e].data();
+      entries[(size_t)e].num_elements = sizes[e][r];
+      entries[(size_t)e].dtype = HOROVOD_FLOAT32;
+    }
+    op.MemcpyInFusionBuffer(entries, displ.data(), r, 4, buffer_data);
+  }
+  op.MemcpyOutFusionBuffer(cof_p.data(), csz_p.data(), buffer_data, 4, ranks, entries);
+  rig.context.StreamSynchronize(rig.context.streams[0][0]);
+  for (int e = 0; e < n; ++e) {
+    size_t at = 0;
+    for (int r = 0; r < ranks; ++r)
+      for (float x : tensors[(size_t)r][(size_t)e]) REQUIRE(outputs[(size_t)e][at++] == x);
+    REQUIRE(at == outputs[(size_t)e].size());
+  }
+}
+
 }  // namespace
 
 int main() {
@@ -414,6 +473,7 @@ int main() {
   elastic_and_timeline();
   fusion_buffer_outlives_its_manager_entry();
   waits_for_the_producer();
+  allgather_hooks();
   std::printf("finalizer ok\n");
   return 0;
 }

@@ -7,7 +7,8 @@ sources are compiled with -fsanitize=thread against tests/native/fake_hvdhip.cc,
 of the C ABI (streams are worker threads, kernels are closures on host memory), and driven by
 tests/native/finalizer_stress.cc: 300 responses over two slots with results checked, two responses
 in flight at once, a failed event wait reaching every callback, inline completion without threads,
-asynchronous completion, elastic polling with the timeline's events, and the pool's own semantics.
+asynchronous completion, elastic polling with the timeline's events, the pool's own semantics, the
+wait for tensors that another stream produces, and the allgather op's fusion-buffer offsets and copies.
 ThreadSanitizer cannot run with the real device runtime (it does not find the GPU under the
 sanitizer's memory layout), which is why the device is modelled."""
 import os
