@@ -139,3 +139,51 @@ def test_timer_measures_stream_time(gpu):
     ms = t.elapsed_ms()
     assert 0.0 < ms < 1000.0
     t.destroy()
+
+
+def test_a_callers_stream_is_forgotten_and_usable_again(gpu, orc):
+    """hvdhip_stream_forget on a stream that the caller owns (torch's here): work queued on it
+    finishes first, the stream's pooled events go, and the entry points that remember streams
+    (pooled events, cached copy tables, the single-layer Adasum plans) work on it afterwards as on a
+    stream they have never seen."""
+    import horovod_amd
+    import torch
+    from oracle_util import F32
+    L = horovod_amd.lib()
+    side = torch.cuda.Stream()
+    s = horovod_amd.Stream(side.cuda_stream)
+    rng = np.random.default_rng(5)
+    sizes = [int(x) for x in rng.integers(1, 200000, 300)]
+    offs = np.concatenate([[0], np.cumsum([(x + 15) // 16 * 16 for x in sizes])]).astype(np.int64)
+    host = rng.integers(0, 256, int(offs[-1]), dtype=np.uint8)
+    src = gpu.upload(host)
+    a = rng.standard_normal(50001).astype(np.float32)
+    b = rng.standard_normal(50001).astype(np.float32)
+    d_a, d_b = gpu.upload(a), gpu.upload(b)
+    n = ctypes.c_int()
+    for rep in range(2):
+        dst = gpu.empty(int(offs[-1]), fill=0)
+        torch.cuda.synchronize()
+        ev = ctypes.c_void_p()
+        horovod_amd.check(L.hvdhip_event_acquire(s.handle, ctypes.byref(ev)), "acquire")
+        L.hvdhip_event_pool_size(s.handle, ctypes.byref(n))
+        assert n.value == 127  # a fresh pool both times
+        gpu.H.batched_d2d_memcpy([dst.data_ptr() + int(o) for o in offs[:-1]],
+                                 [src.data_ptr() + int(o) for o in offs[:-1]], sizes, s)
+        horovod_amd.check(L.hvdhip_event_record(ev, s.handle), "record")
+        dot, an, bn = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+        horovod_amd.check(L.hvdhip_adasum_dot_and_norm_sqrds(d_a.data_ptr(), d_b.data_ptr(), F32, a.size,
+                                                             ctypes.byref(dot), ctypes.byref(an), ctypes.byref(bn),
+                                                             s.handle), "dot")
+        assert np.allclose([dot.value, an.value, bn.value], orc.adasum_dot_norms(a, b, F32), rtol=1e-12, atol=0)
+        # one more copy left queued: forget waits for it
+        gpu.H.batched_d2d_memcpy([dst.data_ptr() + int(o) for o in offs[:-1]],
+                                 [src.data_ptr() + int(o) for o in offs[:-1]], sizes, s)
+        horovod_amd.check(L.hvdhip_event_release(s.handle, ev), "release")
+        horovod_amd.check(L.hvdhip_stream_forget(s.handle), "forget")
+        assert side.query()  # nothing left running on the stream
+        L.hvdhip_event_pool_size(s.handle, ctypes.byref(n))
+        assert n.value == 0
+        out = dst.cpu().numpy()
+        for o, x in zip(offs[:-1], sizes):
+            assert np.array_equal(out[o:o + x], host[o:o + x])
